@@ -47,6 +47,7 @@ class StateView:
     """What a stateful mixer gets: ``state[slot]`` is a request's state in this layer."""
     state: torch.Tensor      # [num_slots, *shape]
     write: bool
+    extra: Optional[Dict[str, torch.Tensor]] = None     # the need's further tensors, [num_slots, *shape] each
 
 
 class PageGroup:
@@ -106,7 +107,8 @@ class CacheManager:
         self.groups: List[PageGroup] = []
         self._where: Dict[int, Tuple[str, int, int]] = {}     # cache id -> (kind, group/tensor, layer slot)
         by_need: Dict[PagedKVNeed, List[int]] = {}
-        self.state_tensors: Dict[int, torch.Tensor] = {}
+        self.state_tensors: Dict[object, torch.Tensor] = {}      # cache id (or (cache id, name) of a further tensor) -> [slots, ...]
+        self._state_extra: Dict[int, List[str]] = {}
         for cid in sorted(needs):
             need = needs[cid]
             if isinstance(need, PagedKVNeed):
@@ -115,8 +117,10 @@ class CacheManager:
                 self._where[cid] = ("state", cid, 0)
                 if device is not None:
                     # one slot more than requests: the scratch slot of rows that belong to no request
-                    self.state_tensors[cid] = torch.zeros((max_requests + 1,) + tuple(need.shape),
-                                                          device=device, dtype=need.dtype)
+                    for name, shape, state_dtype in need.all_tensors():
+                        self.state_tensors[(cid, name) if name else cid] = torch.zeros((max_requests + 1,) + shape,
+                                                                                    device=device, dtype=state_dtype)
+                self._state_extra[cid] = [name for name, _, _ in need.extra]
             else:
                 raise TypeError(f"cache {cid}: unknown need {need!r}")
         for gi, (need, cids) in enumerate(by_need.items()):
@@ -163,7 +167,8 @@ class CacheManager:
         if kind == "kv":
             g = self.groups[where]
             return KVCacheView(g.k_pool[slot], g.v_pool[slot], g.index, g.page_size, write)
-        return StateView(self.state_tensors[where], write)
+        names = self._state_extra.get(where) or []
+        return StateView(self.state_tensors[where], write, {n: self.state_tensors[(where, n)] for n in names} if names else None)
 
     # -- life of a request -----------------------------------------------------
     def add_request(self, rid) -> int:

@@ -715,3 +715,207 @@ class BeloraxConfig(ModelConfig):
         if self.eos_token_ids:
             d["eos_token_id"] = list(self.eos_token_ids)
         return d
+
+
+# ---------------------------------------------------------------------------
+# Pilavik: a norm before and after every sub-layer, a gate on each sub-layer's result, a stretch
+# of layers that runs several times
+# ---------------------------------------------------------------------------
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """Mixer ``delta``: the gated delta rule on ``heads`` value heads of ``vdim`` that share ``kv_heads``
+    query/key heads of ``dim``; q, k, v pass a causal convolution of ``conv`` taps."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    kind: str = "delta"
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "GatedDeltaSpec":
+        s = GatedDeltaSpec(heads=_require(m, "heads", int, where), kv_heads=_require(m, "kv_heads", int, where),
+                           dim=_require(m, "dim", int, where), vdim=_require(m, "vdim", int, where),
+                           conv=_require(m, "conv", int, where))
+        if min(s.heads, s.kv_heads, s.dim, s.vdim, s.conv) <= 0 or s.heads % s.kv_heads:
+            raise ConfigError(f"{where}: heads, kv_heads, dim, vdim and conv must be > 0 and heads a multiple of kv_heads")
+        if s.dim > MAX_HEAD_DIM or s.conv > 8:
+            raise ConfigError(f"{where}: dim {s.dim} exceeds {MAX_HEAD_DIM}, the most key rows the state kernel takes, "
+                              f"or conv {s.conv} exceeds the 8 taps the convolution kernel takes")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "conv": self.conv}
+
+
+@dataclass(frozen=True)
+class SinkLatentAttentionSpec:
+    """Mixer ``latent_attention`` of this design: keys and values from one latent a token (see
+    ``LatentAttentionSpec``), an unstretched interleaved rotation, a sliding window of ``window`` positions
+    (None: all) and a learned sink a head in the softmax's denominator."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
+    rot_base: float
+    rot_dims: int
+    window: Optional[int] = None
+    kind: str = "latent_attention"
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "SinkLatentAttentionSpec":
+        base, dims, scaling = _rot_of(m, where)
+        if scaling is not None:
+            raise ConfigError(f"{where}.rot: this design's rotation is not stretched")
+        mask = m.get("mask")
+        if mask is not None and not isinstance(mask, dict):
+            raise ConfigError(f"{where}: 'mask' must be an object or null")
+        window = _require(mask, "size", int, where + ".mask") if mask is not None else None
+        s = SinkLatentAttentionSpec(
+            heads=_require(m, "heads", int, where), dim=_require(m, "dim", int, where),
+            rot_dim=_require(m, "rot_dim", int, where), vdim=_require(m, "vdim", int, where),
+            kv_rank=_require(m, "kv_rank", int, where), scale=_require(m, "scale", float, where),
+            rot_base=base, rot_dims=dims, window=window)
+        if min(s.heads, s.dim, s.rot_dim, s.vdim, s.kv_rank) <= 0 or (window is not None and window <= 0):
+            raise ConfigError(f"{where}: heads, dim, rot_dim, vdim, kv_rank and mask.size must be > 0")
+        if s.rot_dims > s.rot_dim:
+            raise ConfigError(f"{where}: rot.dims {s.rot_dims} exceeds rot_dim {s.rot_dim}")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        d = {"heads": self.heads, "dim": self.dim, "rot_dim": self.rot_dim, "vdim": self.vdim, "kv_rank": self.kv_rank,
+             "scale": self.scale, "rot": _rot_dict(self.rot_base, self.rot_dims)}
+        if self.window is not None:
+            d["mask"] = {"size": self.window}
+        return d
+
+
+PILAVIK_MIXERS = {"delta": GatedDeltaSpec, "latent_attention": SinkLatentAttentionSpec}
+
+
+@dataclass(frozen=True)
+class PilavikFeedForwardSpec:
+    """``dense``: one feed-forward of width ``ff`` (biases, an activation that norms powers).  ``moe``:
+    ``experts`` gated feed-forwards of width ``ff`` of which a token uses ``top``, weights times
+    ``router_scale``, and a shared one of width ``shared_ff`` (0: none) for every token."""
+    kind: str
+    ff: int
+    experts: int = 0
+    top: int = 0
+    router_scale: float = 1.0
+    shared_ff: int = 0
+
+    @staticmethod
+    def from_dict(mlp: Dict[str, Any], where: str) -> "PilavikFeedForwardSpec":
+        kind = _require(mlp, "kind", str, where)
+        if kind == "dense":
+            s = PilavikFeedForwardSpec("dense", _require(mlp, "ff", int, where))
+        elif kind == "moe":
+            router = _obj(mlp, "router", where)
+            shared = mlp.get("shared")
+            if shared is not None and not isinstance(shared, dict):
+                raise ConfigError(f"{where}: 'shared' must be an object or null")
+            s = PilavikFeedForwardSpec(
+                "moe", _require(_obj(mlp, "expert", where), "ff", int, where + ".expert"),
+                _require(router, "experts", int, where + ".router"), _require(router, "top", int, where + ".router"),
+                _typed(router.get("scale", 1.0), "scale", float, where + ".router"),
+                _require(shared, "ff", int, where + ".shared") if shared is not None else 0)
+            if not (0 < s.top <= s.experts) or s.experts > 512 or s.shared_ff < 0:
+                raise ConfigError(f"{where}: need 0 < top <= experts <= 512 and shared.ff >= 0")
+        else:
+            raise ConfigError(f"{where}: unknown feed-forward kind {kind!r} (known: dense, moe)")
+        if s.ff <= 0:
+            raise ConfigError(f"{where}: ff must be > 0")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        if self.kind == "dense":
+            return {"kind": "dense", "ff": self.ff}
+        d = {"kind": "moe", "expert": {"ff": self.ff},
+             "router": {"experts": self.experts, "top": self.top, "scale": self.router_scale}}
+        if self.shared_ff:
+            d["shared"] = {"ff": self.shared_ff}
+        return d
+
+
+@dataclass(frozen=True)
+class PilavikLayer:
+    mixer: Any                                       # one of the specs above
+    mlp: Optional[PilavikFeedForwardSpec] = None     # None: the layer has no feed-forward
+
+    @property
+    def type(self) -> str:
+        return self.mixer.kind
+
+
+@dataclass(frozen=True)
+class PilavikConfig(ModelConfig):
+    """``{"architecture": "Pilavik", "vocab", "width", "norm": {"eps"}, "layers": [{"type", "mixer": {...},
+    "mlp": {...} | null}], "loop": {"start", "stop", "times"} | absent}``.  Layers ``start .. stop - 1`` run
+    ``times`` times in a row with the same weights, each pass on a cache or state of its own; the head has
+    a matrix of its own; no end-of-sequence token of its own."""
+
+    vocab_size: int = 0
+    hidden_size: int = 0
+    norm_eps: float = 1e-6
+    layers: tuple = ()
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1          # 1 with loop_start == loop_stop: no loop
+    eos_token_ids: tuple = ()
+    architecture: str = "Pilavik"
+
+    @property
+    def has_loop(self) -> bool:
+        return self.loop_stop > self.loop_start
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any], where: str = "config.json") -> "PilavikConfig":
+        layers_in = d.get("layers")
+        if not isinstance(layers_in, list) or not layers_in:
+            raise ConfigError(f"{where}: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(layers_in):
+            w = f"{where}.layers[{i}]"
+            if not isinstance(entry, dict):
+                raise ConfigError(f"{w}: must be an object")
+            kind = _require(entry, "type", str, w)
+            if kind not in PILAVIK_MIXERS:
+                raise ConfigError(f"{w}: unknown mixer type {kind!r} (known: {', '.join(sorted(PILAVIK_MIXERS))})")
+            mixer = PILAVIK_MIXERS[kind].from_dict(_obj(entry, "mixer", w), w + ".mixer")
+            mlp = entry.get("mlp")
+            if mlp is not None and not isinstance(mlp, dict):
+                raise ConfigError(f"{w}: 'mlp' must be null or an object")
+            layers.append(PilavikLayer(mixer, PilavikFeedForwardSpec.from_dict(mlp, w + ".mlp") if mlp is not None else None))
+        loop = d.get("loop")
+        start = stop = 0
+        times = 1
+        if loop is not None:
+            if not isinstance(loop, dict):
+                raise ConfigError(f"{where}: 'loop' must be an object or null")
+            w = where + ".loop"
+            start, stop, times = _require(loop, "start", int, w), _require(loop, "stop", int, w), _require(loop, "times", int, w)
+            if not (0 <= start <= stop <= len(layers)) or times < 1:
+                raise ConfigError(f"{w}: need 0 <= start <= stop <= {len(layers)} layers and times >= 1")
+        eos = d.get("eos_token_id")
+        eos_ids = () if eos is None else tuple(_typed(e, "eos_token_id", int, where) for e in (eos if isinstance(eos, list) else [eos]))
+        cfg = cls(vocab_size=_require(d, "vocab", int, where), hidden_size=_require(d, "width", int, where),
+                  norm_eps=_require(_obj(d, "norm", where), "eps", float, where + ".norm"),
+                  layers=tuple(layers), loop_start=start, loop_stop=stop, loop_times=times, eos_token_ids=eos_ids)
+        if cfg.vocab_size <= 0 or cfg.hidden_size <= 0 or not cfg.norm_eps > 0:
+            raise ConfigError(f"{where}: vocab and width must be > 0, norm.eps > 0")
+        return cfg
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {
+            "architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+            "norm": {"eps": self.norm_eps},
+            "layers": [{"type": l.type, "mixer": l.mixer.to_dict(), "mlp": None if l.mlp is None else l.mlp.to_dict()}
+                       for l in self.layers]}
+        if self.has_loop:
+            d["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids)
+        return d

@@ -102,3 +102,4 @@ def _ensure_builtin() -> None:
     from ..models import llama  # noqa: F401  (registers LlamaForCausalLM)
     from ..models import tedelix  # noqa: F401  (registers Tedelix)
     from ..models import belorax  # noqa: F401  (registers Belorax)
+    from ..models import pilavik  # noqa: F401  (registers Pilavik)

@@ -117,6 +117,16 @@ __device__ __forceinline__ void aw_merge(float& m, float& l, float (&acc)[NC], f
     m = M;
 }
 
+// What a row's sums are multiplied by at the end: 1 / l, or, with a sink (a learned score that has no
+// key and no value and counts once in the denominator), exp(m - M) / (l exp(m - M) + exp(sink - M)) with
+// M = max(m, sink).  0 where nothing was seen.
+__device__ __forceinline__ float aw_final_factor(float m, float l, const float* __restrict__ sink, int head) {
+    if (!(l > 0.f)) return 0.f;
+    if (sink == nullptr) return 1.f / l;
+    const float s = sink[head], M = fmaxf(m, s), a = expf(m - M);
+    return a / (l * a + expf(s - M));
+}
+
 // 16 bytes of the cache as 32-bit values: 4 floats or 8 bfloat16
 __device__ __forceinline__ void ld_vec16(const float* p, float* f) {
     const float4 v = *reinterpret_cast<const float4*>(p);
@@ -136,7 +146,7 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
         const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int num_rows, int H, int Hkv, int dk, int dv, int page, float scale, int window, int TQ, int NK,
-        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved) {
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved, const float* __restrict__ sink) {
     extern __shared__ __align__(16) float lds[];
     const int dkp = (dk + 3) & ~3, ks_stride = dkp + 4, vs_stride = dv + 1;
     float* Qs = lds;                                   // [AW_ROWS][dkp]
@@ -316,10 +326,11 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
             const int r = wave + 4 * i;
             if (r >= R) continue;
             T* o = out + (size_t)(t0 + r / G) * out_stride + (g * G + r % G) * dv;
+            const float fin = sink ? aw_final_factor(m[i], l[i], sink, g * G + r % G) : 0.f;
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 const int d = lane + 64 * c;
-                if (d < dv) st_f32(o + d, l[i] > 0.f ? acc[i][c] / l[i] : 0.f);
+                if (d < dv) st_f32(o + d, sink ? acc[i][c] * fin : (l[i] > 0.f ? acc[i][c] / l[i] : 0.f));
             }
         }
         return;
@@ -334,7 +345,7 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int d = lane + 64 * c;
-            if (d < dv) Os[r * dv + d] = l[i] > 0.f ? acc[i][c] / l[i] : 0.f;
+            if (d < dv) Os[r * dv + d] = sink ? acc[i][c] * aw_final_factor(m[i], l[i], sink, g * G + r % G) : (l[i] > 0.f ? acc[i][c] / l[i] : 0.f);
         }
     }
     __syncthreads();
@@ -360,7 +371,7 @@ __global__ __launch_bounds__(64) void attn_window_combine_kernel(
         const float* __restrict__ part_ml, const float* __restrict__ part_o, T* __restrict__ out, int out_stride,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int H, int dv, int window, int NK, int slots,
-        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved) {
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved, const float* __restrict__ sink) {
     __shared__ float Os[256];
     const int b = blockIdx.y, h = blockIdx.x, lane = threadIdx.x;
     const int t = cu_q[b];
@@ -399,7 +410,7 @@ __global__ __launch_bounds__(64) void attn_window_combine_kernel(
     for (int c = 0; c < NC; ++c) {
         const int d = lane + 64 * c;
         if (d < dv) {
-            const float y = l > 0.f ? acc[c] / l : 0.f;
+            const float y = sink ? acc[c] * aw_final_factor(m, l, sink, h) : (l > 0.f ? acc[c] / l : 0.f);
             if (vcos == nullptr) st_f32(o + d, y);
             else Os[d] = y;
         }
@@ -624,7 +635,7 @@ template <typename T>
 int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
               const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
               int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved,
-              int slots, float* workspace, hipStream_t stream) {
+              int slots, float* workspace, const float* sink, hipStream_t stream) {
     const int G = H / Hkv, TQ = AW_ROWS / G;
     const int NK = aw_keys_a_block(dk, dv);
     const size_t lds = aw_lds_bytes(dk, dv, NK);
@@ -656,12 +667,12 @@ int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, con
         auto combine = NC == 1 ? attn_window_combine_kernel<T, 1> : NC == 2 ? attn_window_combine_kernel<T, 2>
                      : NC == 3 ? attn_window_combine_kernel<T, 3> : attn_window_combine_kernel<T, 4>;
         combine<<<dim3(H, num_rows), 64, 0, stream>>>(part_ml, part_o, out, out_stride, cu_q, q_start, kv_lens, H, dv, window, AD_KEYS, slots,
-                                                      vcos, vsin, v_interleaved);
+                                                      vcos, vsin, v_interleaved, sink);
         return 0;
     }
     const int tiles = (Tn + TQ - 1) / TQ + num_rows;   // at most: every request may end in a short tile
     kernel<<<dim3(tiles, Hkv), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens,
-                                                   num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin, v_interleaved);
+                                                   num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin, v_interleaved, sink);
     return 0;
 }
 }  // namespace
@@ -675,6 +686,7 @@ extern "C" size_t ri_attention_window_workspace(int T, int H, int dk, int dv, in
 
 // Attention of the step's tokens (rotated queries in q) over the cache; out [T][>= H dv].
 // vcos / vsin [positions][dv / 2]: the sums are turned back by the query's position (null: not).
+// sink [H] (null: none): a score a query head that counts once in the softmax's denominator.
 // single_tokens != 0: every row of the step has at most one token and row b's token is token
 // cu_q[b]; with a workspace of ri_attention_window_workspace floats the keys of a row are then
 // divided between blocks (the same bits as without).
@@ -683,7 +695,7 @@ extern "C" int ri_attention_window(
         int num_pages, int page, int H, int Hkv, int dk, int dv, const int* table, int max_blocks,
         const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int T,
         float scale, int window, const float* vcos, const float* vsin, int v_table_rows, int v_interleaved,
-        int single_tokens, int max_kv_len, float* workspace, size_t workspace_floats, hipStream_t stream) {
+        int single_tokens, int max_kv_len, float* workspace, size_t workspace_floats, const float* sink, hipStream_t stream) {
     RI_REQUIRE(ri_attention_window_supported(H, Hkv, dk, dv), "ri_attention_window: sizes not taken (H=%d Hkv=%d dk=%d dv=%d)", H, Hkv, dk, dv);
     RI_REQUIRE(T >= 0 && num_rows >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0 && page > 0, "ri_attention_window: bad sizes");
     RI_REQUIRE(q_stride >= H * dk && out_stride >= H * dv, "ri_attention_window: row strides too small");
@@ -700,9 +712,9 @@ extern "C" int ri_attention_window(
     }
     int rc;
     if (dtype == RI_F32)
-        rc = aw_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, stream);
+        rc = aw_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, sink, stream);
     else if (dtype == RI_BF16)
-        rc = aw_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, stream);
+        rc = aw_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, sink, stream);
     else
         return ri_fail("ri_attention_window: unknown dtype %d", dtype);
     if (rc) return rc;
@@ -743,7 +755,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(
         const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int num_rows, int H, int Hkv, int dk, int dv, int page, float scale, int window,
-        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved) {
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved, const float* __restrict__ sink) {
     extern __shared__ __align__(16) float lds[];
     constexpr int DKP = 8 * QU, KS = DKP + 4;
     const int vs_stride = dv + 8;
@@ -916,7 +928,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(
     }
     // the sums of a query lie in the lane of its lower and of its upper half: add the two l
     l += __shfl_xor(l, 32, 64);
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const float inv = aw_final_factor(m, l, sink, head);
     __syncthreads();                                   // the last keys and values have been used
     float* ow = Os + (size_t)wave * 32 * dv;
     if (wave_on) {
@@ -951,7 +963,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(
 template <typename T, int QU, int FT>
 int am_launch_as(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
                  const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
-                 int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, hipStream_t stream) {
+                 int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, const float* sink, hipStream_t stream) {
     const int G = H / Hkv, HB = G < 4 ? G : 4, SB = 4 / HB, TQB = 32 * SB;
     const size_t lds = am_lds_bytes(QU, dv);
     auto kernel = attn_window_mfma_kernel<T, QU, FT>;
@@ -965,16 +977,16 @@ int am_launch_as(const T* q, int q_stride, T* out, int out_stride, const T* kc, 
     }
     const int tiles = (Tn + TQB - 1) / TQB + num_rows;
     kernel<<<dim3(tiles, Hkv, (G + 3) / 4), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start,
-                                                               kv_lens, num_rows, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved);
+                                                               kv_lens, num_rows, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink);
     return 0;
 }
 
 template <typename T>
 int am_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
               const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
-              int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, hipStream_t stream) {
+              int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, const float* sink, hipStream_t stream) {
 #define RI_AM(QU, FT) return am_launch_as<T, QU, FT>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens, \
-        num_rows, Tn, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream)
+        num_rows, Tn, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, stream)
     if (dk <= 64) { if (dv <= 64) RI_AM(8, 2); if (dv <= 128) RI_AM(8, 4); RI_AM(8, 8); }
     if (dk <= 128) { if (dv <= 64) RI_AM(16, 2); if (dv <= 128) RI_AM(16, 4); RI_AM(16, 8); }
     if (dv <= 64) RI_AM(32, 2);
@@ -998,7 +1010,7 @@ extern "C" int ri_attention_window_mfma(
         int num_pages, int page, int H, int Hkv, int dk, int dv, const int* table, int max_blocks,
         const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int T,
         float scale, int window, const float* vcos, const float* vsin, int v_table_rows, int v_interleaved,
-        hipStream_t stream) {
+        const float* sink, hipStream_t stream) {
     RI_REQUIRE(ri_attention_window_mfma_supported(H, Hkv, dk, dv), "ri_attention_window_mfma: sizes not taken (H=%d Hkv=%d dk=%d dv=%d)", H, Hkv, dk, dv);
     RI_REQUIRE(T >= 0 && num_rows >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0 && page > 0, "ri_attention_window_mfma: bad sizes");
     RI_REQUIRE(q_stride >= H * dk && out_stride >= H * dv, "ri_attention_window_mfma: row strides too small");
@@ -1008,9 +1020,9 @@ extern "C" int ri_attention_window_mfma(
     RI_REQUIRE(Hkv <= 65535, "ri_attention_window_mfma: too many key/value heads for the grid");
     int rc;
     if (dtype == RI_F32)
-        rc = am_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream);
+        rc = am_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, stream);
     else if (dtype == RI_BF16)
-        rc = am_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, stream);
+        rc = am_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, stream);
     else
         return ri_fail("ri_attention_window_mfma: unknown dtype %d", dtype);
     if (rc) return rc;

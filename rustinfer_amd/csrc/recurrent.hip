@@ -8,6 +8,11 @@
 //   delta form:  u_t = k_t / sqrt(|k_t|^2 + unit_eps),  w_t = exp(-c * sigmoid(wl_t + w0)),
 //                a_t = sigmoid(al_t + ab), all per key channel (a generalized delta rule: the
 //                state forgets by w and gives up what it held along u at the rate a).
+//   gated form:  the delta form's walk with one decay and one write strength a head and token
+//                (a gated delta rule: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, which
+//                is w = g, a u = beta g k, and beta k in place of k in the last term): q and k are made
+//                unit vectors (q also times q_scale), beta = sigmoid(bl_t), g = exp(-A softplus(gl_t +
+//                dt_bias)); several heads may share one head of q and k.
 // Both terms of the delta form read the old state.  Everything after the projections is 32-bit.
 //
 // One kernel walks a request's tokens of the step in order; a step of single tokens is the same
@@ -43,7 +48,16 @@ struct ScanArgs {
     const float *rot_cos, *rot_sin;
     int rot;
     float k_scale;
+    // the gated form: wl, al hold one value a head ([T][>= H], 32-bit or bfloat16 by gate_bf16);
+    // w0 = A [H], ab = dt_bias [H]; kv_group heads share a head of r and k; r is multiplied by q_scale
+    int gate_bf16, kv_group;
+    float q_scale;
 };
+
+__device__ __forceinline__ float ld_gate(const void* p, size_t at, int is_bf16) {
+    return is_bf16 ? bf16_to_f32(reinterpret_cast<const bf16_t*>(p)[at]) : reinterpret_cast<const float*>(p)[at];
+}
+__device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
 // exp on the hardware's 2^x (an error of a unit or two in the last place of 32 bits) and a division
 // without the library's special cases: the staging of a stretch is a third of the walk's time
@@ -85,8 +99,9 @@ __device__ __forceinline__ float wave_sum_rows(float x) {
            + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 48))));
 }
 
-template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT>
+template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT, bool GATED = false>
 __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) {
+    static_assert(!GATED || (DELTA && !ROT), "the gated form is a delta form without a rotation");
     constexpr int SC_EPL = EPL;
     extern __shared__ __align__(16) float lds[];
     constexpr int TPW = SC_CH / NW;                    // tokens of a stretch a wave stages
@@ -114,8 +129,10 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
     const T* wlp = (const T*)a.wl; const T* alp = (const T*)a.al;
 
     // what this thread stages of a stretch: asked for a stretch ahead, so that the walk hides the wait
-    float raw_r[TPW][SC_EPL], raw_k[TPW][SC_EPL], raw_w[DELTA ? TPW : 1][SC_EPL], raw_a[DELTA ? TPW : 1][SC_EPL];
+    float raw_r[TPW][SC_EPL], raw_k[TPW][SC_EPL], raw_w[DELTA && !GATED ? TPW : 1][SC_EPL], raw_a[DELTA && !GATED ? TPW : 1][SC_EPL];
     float raw_v[SC_CH];
+    float raw_gb[GATED ? TPW : 1], raw_ga[GATED ? TPW : 1];       // the gated form's two numbers a token
+    const int hk = GATED ? h / a.kv_group : h;                     // the head of r and k this head reads
     // ROT: the rotation partners of r and k (feature idx +- rot/2), asked for with them
     float part_r[ROT ? TPW : 1][SC_EPL], part_k[ROT ? TPW : 1][SC_EPL];
     const int rot_half = ROT ? a.rot >> 1 : 0;
@@ -130,7 +147,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                 const int idx = e * 64 + lane;
                 const bool on = tt < nc && idx < dk;
                 const size_t t = (size_t)(t_lo + c0 + (on ? tt : 0));
-                const int c = h * dk + (on ? idx : 0);
+                const int c = hk * dk + (on ? idx : 0);
                 raw_r[i][e] = on ? ld_f32(rp + t * a.r_stride + c) : 0.f;
                 raw_k[i][e] = on ? ld_f32(kp + t * a.k_stride + c) : 0.f;
                 if (ROT) {
@@ -139,10 +156,15 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                     part_r[i][e] = turn ? ld_f32(rp + t * a.r_stride + cp) : 0.f;
                     part_k[i][e] = turn ? ld_f32(kp + t * a.k_stride + cp) : 0.f;
                 }
-                if (DELTA) {
+                if (DELTA && !GATED) {
                     raw_w[i][e] = on ? ld_f32(wlp + t * a.wl_stride + c) : 0.f;
                     raw_a[i][e] = on ? ld_f32(alp + t * a.al_stride + c) : 0.f;
                 }
+            }
+            if (GATED) {
+                const size_t t = (size_t)(t_lo + c0 + (tt < nc ? tt : 0));
+                raw_gb[i] = ld_gate(a.wl, t * a.wl_stride + h, a.gate_bf16);
+                raw_ga[i] = ld_gate(a.al, t * a.al_stride + h, a.gate_bf16);
             }
         }
 #pragma unroll
@@ -164,7 +186,25 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
         for (int i = 0; i < TPW; ++i) {
             const int tt = wave + i * NW;
             if (tt >= nc) continue;
-            if (DELTA) {
+            if (GATED) {
+                float sk = 0.f, sq = 0.f;
+#pragma unroll
+                for (int e = 0; e < SC_EPL; ++e) { sk = fmaf(raw_k[i][e], raw_k[i][e], sk); sq = fmaf(raw_r[i][e], raw_r[i][e], sq); }
+                sk = wave_sum_rows(sk);
+                sq = wave_sum_rows(sq);
+                const float inv_k = 1.f / sqrtf(sk + a.unit_eps), inv_q = a.q_scale / sqrtf(sq + a.unit_eps);
+                const float beta = 1.f / (1.f + expf(-raw_gb[i]));
+                const float g = expf(-a.w0[h] * softplusf_(raw_ga[i] + a.ab[h]));
+#pragma unroll
+                for (int e = 0; e < SC_EPL; ++e) {
+                    const int idx = e * 64 + lane;
+                    if (idx >= DKP) continue;
+                    const float u = idx < dk ? raw_k[i][e] * inv_k : 0.f;
+                    rs[tt * DKP + idx] = idx < dk ? raw_r[i][e] * inv_q : 0.f;
+                    us[tt * DKP + idx] = u; ks[tt * DKP + idx] = beta * u;
+                    aus[tt * DKP + idx] = beta * g * u; ws[tt * DKP + idx] = g;
+                }
+            } else if (DELTA) {
                 float ssq = 0.f;
 #pragma unroll
                 for (int e = 0; e < SC_EPL; ++e) ssq = fmaf(raw_k[i][e], raw_k[i][e], ssq);
@@ -276,12 +316,12 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
     }
 }
 
-template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT>
+template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT, bool GATED = false>
 int launch_scan_rot(const ScanArgs& a, int num_rows, hipStream_t stream) {
     const int P = a.P, DKP = P * R, CPB = NW * (64 / P);
     const size_t lds = sizeof(float) * 2 * ((DELTA ? 5 : 2) * SC_CH * DKP + SC_CH * CPB);
     dim3 grid((a.dv + CPB - 1) / CPB, a.H, num_rows);
-    auto kernel = linear_scan_kernel<T, DELTA, R, NW, EPL, ROT>;
+    auto kernel = linear_scan_kernel<T, DELTA, R, NW, EPL, ROT, GATED>;
     if (lds > 64 * 1024) {
         // more LDS than a kernel gets unasked (the delta form with more than 128 key rows)
         static bool asked = false;
@@ -295,28 +335,29 @@ int launch_scan_rot(const ScanArgs& a, int num_rows, hipStream_t stream) {
     return 0;
 }
 
-template <typename T, bool DELTA, int R, int NW, int EPL>
+template <typename T, bool DELTA, int R, int NW, int EPL, bool GATED = false>
 int launch_scan_as(const ScanArgs& a, int num_rows, hipStream_t stream) {
+    if constexpr (GATED) return launch_scan_rot<T, true, R, NW, EPL, false, true>(a, num_rows, stream);
     if constexpr (!DELTA) {
         if (a.rot_cos != nullptr || a.k_scale != 1.f) return launch_scan_rot<T, DELTA, R, NW, EPL, true>(a, num_rows, stream);
     }
     return launch_scan_rot<T, DELTA, R, NW, EPL, false>(a, num_rows, stream);
 }
 
-template <typename T, bool DELTA, int R>
+template <typename T, bool DELTA, int R, bool GATED = false>
 int launch_scan(const ScanArgs& a, int num_rows, hipStream_t stream) {
     // Four waves a block share the staging of a stretch (a wave alone spends more instructions on
     // staging than on the walk); one wave where a head has no more than 64 threads.
     const bool four = (long)a.dv * a.P > 64;
     const int epl = (a.dk + 63) / 64;
     if (four) {
-        if (epl == 1) return launch_scan_as<T, DELTA, R, 4, 1>(a, num_rows, stream);
-        if (epl == 2) return launch_scan_as<T, DELTA, R, 4, 2>(a, num_rows, stream);
-        return launch_scan_as<T, DELTA, R, 4, 4>(a, num_rows, stream);
+        if (epl == 1) return launch_scan_as<T, DELTA, R, 4, 1, GATED>(a, num_rows, stream);
+        if (epl == 2) return launch_scan_as<T, DELTA, R, 4, 2, GATED>(a, num_rows, stream);
+        return launch_scan_as<T, DELTA, R, 4, 4, GATED>(a, num_rows, stream);
     }
-    if (epl == 1) return launch_scan_as<T, DELTA, R, 1, 1>(a, num_rows, stream);
-    if (epl == 2) return launch_scan_as<T, DELTA, R, 1, 2>(a, num_rows, stream);
-    return launch_scan_as<T, DELTA, R, 1, 4>(a, num_rows, stream);
+    if (epl == 1) return launch_scan_as<T, DELTA, R, 1, 1, GATED>(a, num_rows, stream);
+    if (epl == 2) return launch_scan_as<T, DELTA, R, 1, 2, GATED>(a, num_rows, stream);
+    return launch_scan_as<T, DELTA, R, 1, 4, GATED>(a, num_rows, stream);
 }
 
 }  // namespace
@@ -356,6 +397,7 @@ extern "C" int ri_linear_scan(
     a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
     a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = silu_in; a.unit_eps = unit_eps; a.decay_c = decay_c;
     a.rot_cos = rot_cos; a.rot_sin = rot_sin; a.rot = rot_cos ? rot : 0; a.k_scale = k_scale;
+    a.gate_bf16 = 0; a.kv_group = 1; a.q_scale = 1.f;
     int rc;
 #define RI_SCAN(TT, DD) (R == 8 ? launch_scan<TT, DD, 8>(a, num_rows, stream) : launch_scan<TT, DD, 16>(a, num_rows, stream))
     if (dtype == RI_F32) rc = delta ? RI_SCAN(float, true) : RI_SCAN(float, false);
@@ -364,6 +406,42 @@ extern "C" int ri_linear_scan(
 #undef RI_SCAN
     if (rc) return rc;
     RI_LAUNCHED("ri_linear_scan");
+    return 0;
+}
+
+// The gated form of the walk.  q, k [T, >= Hk dk] and v [T, >= H dv] are 32-bit (what the short
+// convolutions leave); bl, gl [T, >= H] hold the write strength's and the decay's inputs, one a head, in
+// gate_dtype; A, dt_bias [H] 32-bit: g = exp(-A softplus(gl + dt_bias)), beta = sigmoid(bl).  Head h reads
+// q/k head h / (H / Hk).  q and k are divided by sqrt(|.|^2 + unit_eps), q also times q_scale.
+extern "C" int ri_gated_delta_scan(
+        const float* q, int q_stride, const float* k, int k_stride, const float* v, int v_stride,
+        const void* bl, int bl_stride, const void* gl, int gl_stride, int gate_dtype,
+        const float* A, const float* dt_bias, float unit_eps, float q_scale,
+        float* state, int num_slots, float* out, int out_stride,
+        const int* cu_q, const int* q_start, const int* slots, int num_rows, int T,
+        int H, int Hk, int dk, int dv, hipStream_t stream) {
+    RI_REQUIRE(H > 0 && Hk > 0 && H % Hk == 0 && dk > 0 && dv > 0 && dk <= 256, "ri_gated_delta_scan: bad sizes H=%d Hk=%d dk=%d dv=%d (dk <= 256)", H, Hk, dk, dv);
+    RI_REQUIRE(num_rows >= 0 && T >= 0 && num_slots > 0, "ri_gated_delta_scan: bad counts");
+    RI_REQUIRE(q_stride >= Hk * dk && k_stride >= Hk * dk && v_stride >= H * dv && out_stride >= H * dv && bl_stride >= H && gl_stride >= H,
+               "ri_gated_delta_scan: row strides too small");
+    RI_REQUIRE(gate_dtype == RI_F32 || gate_dtype == RI_BF16, "ri_gated_delta_scan: unknown dtype %d", gate_dtype);
+    if (num_rows == 0 || T == 0) return 0;
+    RI_REQUIRE(q && k && v && bl && gl && A && dt_bias && state && out && cu_q && q_start && slots, "ri_gated_delta_scan: null pointer");
+    RI_REQUIRE(H <= 65535 && num_rows <= 65535, "ri_gated_delta_scan: too many heads or rows for the grid");
+    const int R = dk <= 128 ? 8 : 16;
+    int P = 1;
+    while (P * R < dk) P *= 2;
+    ScanArgs a;
+    a.r = q; a.k = k; a.v = v; a.wl = bl; a.al = gl;
+    a.r_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.wl_stride = bl_stride; a.al_stride = gl_stride;
+    a.w0 = A; a.ab = dt_bias; a.decay = nullptr; a.state = state; a.out = out; a.out_stride = out_stride;
+    a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
+    a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = 0; a.unit_eps = unit_eps; a.decay_c = 0.f;
+    a.rot_cos = nullptr; a.rot_sin = nullptr; a.rot = 0; a.k_scale = 1.f;
+    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale;
+    const int rc = R == 8 ? launch_scan<float, true, 8, true>(a, num_rows, stream) : launch_scan<float, true, 16, true>(a, num_rows, stream);
+    if (rc) return rc;
+    RI_LAUNCHED("ri_gated_delta_scan");
     return 0;
 }
 

@@ -48,10 +48,11 @@ def pages_that_fit(needs, page_size: int, element_size: int, free_bytes: int, me
         if isinstance(need, PagedKVNeed):
             per_page += need.num_kv_heads * (need.head_dim + need.value_dim) * page_size * element_size
         elif isinstance(need, StateNeed):
-            n = 1
-            for d in need.shape:
-                n *= int(d)
-            state += (max_requests + 1) * n * torch.empty((), dtype=need.dtype).element_size()
+            for _, shape, dtype in need.all_tensors():
+                n = 1
+                for d in shape:
+                    n *= int(d)
+                state += (max_requests + 1) * n * torch.empty((), dtype=dtype).element_size()
     if per_page == 0:
         return 1
     budget = max(0, int((free_bytes - (1 << 30)) * mem_fraction) - state)

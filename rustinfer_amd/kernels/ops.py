@@ -948,12 +948,14 @@ def window_attention_supported(H: int, Hkv: int, dk: int, dv: int) -> bool:
 def window_attention(q: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, dk: int, dv: int,
                      k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, page: int,
                      ctx, scale: float, window: int = 0, value_rotary=None,
-                     interleaved_values: bool = False) -> None:
+                     interleaved_values: bool = False, sink: Optional[torch.Tensor] = None) -> None:
     """Attention of the step's tokens (rotated queries ``q [T, H dk]``) over the cache into
     ``out [T, H dv]``: keys of size ``dk``, values of size ``dv``, the last ``window`` positions
     (0: all).  ``value_rotary``: the cached values are turned by their positions, and each sum is
-    turned back by its query's."""
-    _dev(q, out, k_cache, v_cache, block_table)
+    turned back by its query's.  ``sink`` (32-bit, one number a query head): ``exp(sink_h)`` joins the
+    softmax's denominator, with no key and no value."""
+    _dev(q, out, k_cache, v_cache, block_table, sink)
+    _f32_vec(sink, H, "window_attention: the sink")
     _rows2d(q, "q")
     _rows2d(out, "out")
     T = q.shape[0]
@@ -973,7 +975,7 @@ def window_attention(q: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, dk: i
         _check(lib.ri_attention_window_mfma(
             _ptr(q), q.stride(0), _ptr(out), out.stride(0), _dt(q), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], page,
             H, Hkv, dk, dv, _ptr(block_table), block_table.shape[1], _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens),
-            ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)), _stream()))
+            ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)), _ptr(sink), _stream()))
         return
     # a step of single tokens divides each row's keys between blocks, through a workspace
     single, ws, need = int(ctx.max_q_len == 1 and T <= ctx.num_rows), None, 0
@@ -986,7 +988,7 @@ def window_attention(q: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, dk: i
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _dt(q), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], page,
         H, Hkv, dk, dv, _ptr(block_table), block_table.shape[1], _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens),
         ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)),
-        single, int(ctx.max_kv_len), _ptr(ws), ctypes.c_size_t(need), _stream()))
+        single, int(ctx.max_kv_len), _ptr(ws), ctypes.c_size_t(need), _ptr(sink), _stream()))
 
 
 # ---------------------------------------------------------------------------
@@ -1161,41 +1163,223 @@ def head_linear(x: torch.Tensor, x_head: int, w: torch.Tensor, out: torch.Tensor
 # ---------------------------------------------------------------------------
 # a feed-forward of many experts
 # ---------------------------------------------------------------------------
-def moe_route(logits: torch.Tensor, weights: torch.Tensor, top: int, renormalize: bool = False) -> None:
+def _score_kind(score: str) -> int:
+    if score not in ("softmax", "sigmoid"):
+        raise KernelError(f"a router scores with 'softmax' or 'sigmoid', got {score!r}")
+    return int(score == "sigmoid")
+
+
+def _moe_widths(gate_up, act, E: int, F: int, shared: int, who: str):
+    """The activations' width: the experts' ``E F`` columns, a shared expert's ``shared`` and zeros up to
+    what ``act`` has."""
+    T, width = gate_up.shape[0], act.shape[1]
+    if gate_up.shape[1] != 2 * E * F + 2 * shared or act.shape[0] != T or width < E * F + shared or act.dtype != gate_up.dtype:
+        raise KernelError(f"{who}: gate_up [T, {2 * E * F + 2 * shared}] and act [T, >= {E * F + shared}] of one dtype expected")
+    return T, width
+
+
+def moe_route(logits: torch.Tensor, weights: torch.Tensor, top: int, renormalize: bool = False,
+              score: str = "softmax", norm_eps: float = 0.0, scale: float = 1.0) -> None:
     """``weights [T, E]`` (32-bit): ``softmax(logits)`` at the ``top`` largest entries of every row (ties:
-    the lower index), 0 elsewhere; ``renormalize`` divides them by their sum."""
+    the lower index), 0 elsewhere; ``renormalize`` divides them by their sum (+ ``norm_eps``).
+    ``score = "sigmoid"``: the scores are ``sigmoid(logits)``, each on its own; ``scale`` multiplies the weights."""
     _dev(logits, weights)
     _rows2d(logits, "logits")
     T, E = logits.shape
     if logits.dtype != torch.float32 or weights.dtype != torch.float32 or tuple(weights.shape) != (T, E) or not weights.is_contiguous():
         raise KernelError("moe_route: 32-bit logits [T, E] and contiguous 32-bit weights [T, E] expected")
-    _check(_lib().ri_moe_route(_ptr(logits), logits.stride(0), _ptr(weights), T, E, int(top), int(bool(renormalize)), _stream()))
+    _check(_lib().ri_moe_route_as(_ptr(logits), logits.stride(0), _ptr(weights), T, E, int(top), int(bool(renormalize)),
+                                  _score_kind(score), ctypes.c_float(norm_eps), ctypes.c_float(scale), _stream()))
 
 
-def moe_swiglu_weighted(gate_up: torch.Tensor, weights: torch.Tensor, act: torch.Tensor, E: int, F: int) -> None:
-    """``act[t, e F + i] = weights[t, e] * silu(gate_up[t, e 2F + i]) * gate_up[t, e 2F + F + i]``."""
+def moe_swiglu_weighted(gate_up: torch.Tensor, weights: torch.Tensor, act: torch.Tensor, E: int, F: int,
+                        shared: int = 0) -> None:
+    """``act[t, e F + i] = weights[t, e] * silu(gate_up[t, e 2F + i]) * gate_up[t, e 2F + F + i]``.
+    ``shared`` > 0: ``gate_up`` has ``2 shared`` more columns, a shared expert's gate and up, and ``act`` gets
+    ``silu(gate) * up`` of them behind the experts' columns (weight 1); wider ``act``: zeros beyond."""
     _dev(gate_up, weights, act)
     _rows2d(gate_up, "gate_up")
     _rows2d(act, "act")
-    T = gate_up.shape[0]
-    if gate_up.shape[1] != 2 * E * F or tuple(act.shape) != (T, E * F) or act.dtype != gate_up.dtype \
-            or weights.dtype != torch.float32 or tuple(weights.shape) != (T, E) or not weights.is_contiguous():
-        raise KernelError("moe_swiglu_weighted: gate_up [T, 2 E F], 32-bit weights [T, E] and act [T, E F] expected")
-    _check(_lib().ri_moe_swiglu_weighted(_ptr(gate_up), gate_up.stride(0), _ptr(weights), _ptr(act), act.stride(0),
-                                         _dt(act), T, E, F, _stream()))
+    T, width = _moe_widths(gate_up, act, E, F, shared, "moe_swiglu_weighted")
+    if weights.dtype != torch.float32 or tuple(weights.shape) != (T, E) or not weights.is_contiguous():
+        raise KernelError("moe_swiglu_weighted: contiguous 32-bit weights [T, E] expected")
+    _check(_lib().ri_moe_swiglu_weighted_shared(_ptr(gate_up), gate_up.stride(0), _ptr(weights), _ptr(act), act.stride(0),
+                                                _dt(act), T, E, F, int(shared), width, _stream()))
 
 
 def moe_swiglu_routed(gate_up: torch.Tensor, logits: torch.Tensor, act: torch.Tensor, E: int, F: int, top: int,
-                      renormalize: bool = False) -> None:
+                      renormalize: bool = False, score: str = "softmax", norm_eps: float = 0.0, scale: float = 1.0,
+                      shared: int = 0) -> None:
     """``moe_route`` and ``moe_swiglu_weighted`` in one launch: the weights are made from the 32-bit
     ``logits [T, E]`` on the way and never stored."""
     _dev(gate_up, logits, act)
     _rows2d(gate_up, "gate_up")
     _rows2d(act, "act")
     _rows2d(logits, "logits")
-    T = gate_up.shape[0]
-    if gate_up.shape[1] != 2 * E * F or tuple(act.shape) != (T, E * F) or act.dtype != gate_up.dtype \
-            or logits.dtype != torch.float32 or tuple(logits.shape) != (T, E):
-        raise KernelError("moe_swiglu_routed: gate_up [T, 2 E F], 32-bit logits [T, E] and act [T, E F] expected")
-    _check(_lib().ri_moe_swiglu_routed(_ptr(gate_up), gate_up.stride(0), _ptr(logits), logits.stride(0), _ptr(act),
-                                       act.stride(0), _dt(act), T, E, F, int(top), int(bool(renormalize)), _stream()))
+    T, width = _moe_widths(gate_up, act, E, F, shared, "moe_swiglu_routed")
+    if logits.dtype != torch.float32 or tuple(logits.shape) != (T, E):
+        raise KernelError("moe_swiglu_routed: 32-bit logits [T, E] expected")
+    _check(_lib().ri_moe_swiglu_routed_as(_ptr(gate_up), gate_up.stride(0), _ptr(logits), logits.stride(0), _ptr(act),
+                                          act.stride(0), _dt(act), T, E, F, int(top), int(bool(renormalize)),
+                                          _score_kind(score), ctypes.c_float(norm_eps), ctypes.c_float(scale),
+                                          int(shared), width, _stream()))
+
+
+# ---------------------------------------------------------------------------
+# layer norm around gated sub-layers, a feed-forward that norms powers, a short convolution, the gated delta rule
+# ---------------------------------------------------------------------------
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, out: torch.Tensor,
+               rows: Optional[torch.Tensor] = None) -> None:
+    """``out = (x - mean) / sqrt(var + eps) * weight + bias`` row by row; ``x`` 32-bit ``[T, d]``; with
+    ``rows`` (int32) only those rows, in that order."""
+    _dev(x, weight, bias, out, rows)
+    T, d = x.shape
+    n_out = rows.numel() if rows is not None else T
+    if rows is not None:
+        _i32(rows, "rows")
+    if x.dtype != torch.float32 or not x.is_contiguous() or tuple(out.shape) != (n_out, d) or not out.is_contiguous():
+        raise KernelError(f"layer_norm: contiguous 32-bit x [T, d] and contiguous out [{n_out}, {d}] expected")
+    _f32_vec(weight, d, "layer_norm: the weight")
+    _f32_vec(bias, d, "layer_norm: the bias")
+    _check(_lib().ri_layer_norm(_ptr(x), _ptr(rows), _ptr(weight), _ptr(bias), ctypes.c_float(eps), _ptr(out), _dt(out),
+                                n_out, d, _stream()))
+
+
+def gated_norm_residual(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float,
+                        gate: Optional[torch.Tensor] = None, gate_bias: Optional[torch.Tensor] = None,
+                        delta_bias: Optional[torch.Tensor] = None, next_norm=None,
+                        next_out: Optional[torch.Tensor] = None) -> None:
+    """``y = (delta + delta_bias) * sigmoid(gate + gate_bias)``; ``x += layer_norm(y) * weight + bias``, in
+    place on the 32-bit stream.  ``delta`` is ``[T, d]`` or a 32-bit stack ``[P, T, d]`` of partial sums;
+    ``gate [T, d]`` may be columns of a wider buffer.  ``next_norm = (weight, bias)`` with ``next_out``
+    ``[T, d]``: the layer norm of the new ``x`` is left there in the same pass."""
+    _dev(x, delta, weight, bias, gate, gate_bias, delta_bias, next_out)
+    T, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("gated_norm_residual: x must be contiguous float32")
+    parts, stride = 1, 0
+    if delta.dim() == 3:
+        parts, stride = delta.shape[0], delta.stride(0)
+    if delta.dim() not in (2, 3) or tuple(delta.shape[-2:]) != (T, d) or delta.stride(-1) != 1 or delta.stride(-2) != d \
+            or (delta.dim() == 3 and delta.dtype != torch.float32):
+        raise KernelError("gated_norm_residual: delta must be [T, d] or a float32 stack [P, T, d] with contiguous rows")
+    for v, name in ((weight, "weight"), (bias, "bias"), (gate_bias, "gate bias"), (delta_bias, "delta bias")):
+        _f32_vec(v, d, f"gated_norm_residual: the {name}")
+    act_dt = _dt(delta) if delta.dtype != torch.float32 else None
+    if gate is not None:
+        _rows2d(gate, "gate")
+        if tuple(gate.shape) != (T, d):
+            raise KernelError(f"gated_norm_residual: gate must be [{T}, {d}]")
+        act_dt = _dt(gate)
+    nw = nb = None
+    if next_out is not None:
+        nw, nb = next_norm
+        _f32_vec(nw, d, "gated_norm_residual: the next norm's weight")
+        _f32_vec(nb, d, "gated_norm_residual: the next norm's bias")
+        if tuple(next_out.shape) != (T, d) or not next_out.is_contiguous():
+            raise KernelError(f"gated_norm_residual: next_out must be contiguous [{T}, {d}]")
+        if gate is not None and next_out.dtype != gate.dtype:
+            raise KernelError("gated_norm_residual: gate and next_out must have one dtype")
+        act_dt = _dt(next_out)
+    if act_dt is None:
+        act_dt = F32
+    _check(_lib().ri_gated_norm_residual(_ptr(x), _ptr(delta), _dt(delta), parts, ctypes.c_longlong(stride), _ptr(delta_bias),
+                                         _ptr(gate), gate.stride(0) if gate is not None else 0, _ptr(gate_bias),
+                                         _ptr(weight), _ptr(bias), ctypes.c_float(eps), _ptr(nw), _ptr(nb), _ptr(next_out),
+                                         act_dt, T, d, _stream()))
+
+
+def stream_add(x: torch.Tensor, other: Optional[torch.Tensor] = None, vec: Optional[torch.Tensor] = None) -> None:
+    """``x[t] += other[t] + vec`` on the 32-bit stream ``[T, d]``; ``other [T, d]`` contiguous, ``vec [d]`` 32-bit."""
+    _dev(x, other, vec)
+    T, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or (other is not None and (tuple(other.shape) != (T, d) or not other.is_contiguous())):
+        raise KernelError("stream_add: contiguous 32-bit x [T, d] and contiguous other [T, d] expected")
+    _f32_vec(vec, d, "stream_add: the vector")
+    _check(_lib().ri_stream_add(_ptr(x), _ptr(other), _dt(other) if other is not None else F32, _ptr(vec), T, d, _stream()))
+
+
+def poly_norm(up: torch.Tensor, bias: Optional[torch.Tensor], coef, eps: float, act: torch.Tensor) -> None:
+    """``act = a N(z) + b N(z^2) + c N(z^3) + e`` with ``z = up + bias``, ``coef = (a, b, c, e)`` and
+    ``N(v) = v / sqrt(mean(v^2) + eps)`` over each row; ``up``, ``act`` ``[T, n]`` (columns of wider buffers allowed)."""
+    _dev(up, bias, act)
+    _rows2d(up, "up")
+    _rows2d(act, "act")
+    T, n = up.shape
+    if tuple(act.shape) != (T, n) or act.dtype != up.dtype:
+        raise KernelError("poly_norm: up and act must be [T, n] of one dtype")
+    _f32_vec(bias, n, "poly_norm: the bias")
+    a, b, c, e = (float(v) for v in coef)
+    _check(_lib().ri_poly_norm(_ptr(up), up.stride(0), _ptr(bias), ctypes.c_float(a), ctypes.c_float(b), ctypes.c_float(c),
+                               ctypes.c_float(e), ctypes.c_float(eps), _ptr(act), act.stride(0), _dt(up), T, n, _stream()))
+
+
+SHORT_CONV_MAX_TAPS = 8
+SHORT_CONV_MAX_SEGMENTS = 4
+
+
+def short_conv(xs, ws, state: Optional[torch.Tensor], out: torch.Tensor, ctx, taps: int, silu: bool = True) -> None:
+    """A causal convolution over time of ``taps`` taps, channel by channel, through the last ``taps - 1``
+    inputs each request keeps in ``state [slots, taps - 1, C]`` (32-bit; a request's first tokens start
+    from zeros): ``xs`` are up to four ``[T, n_s]`` inputs (columns of a wider buffer allowed), ``ws`` their
+    weights ``[n_s, taps]`` (the last column is the current token's); ``out [T, C]`` (32-bit, ``C`` the sum
+    of the ``n_s``) takes the results side by side, through silu if asked."""
+    _dev(state, out, *xs, *ws)
+    if not xs or len(xs) != len(ws) or len(xs) > SHORT_CONV_MAX_SEGMENTS:
+        raise KernelError(f"short_conv: 1 to {SHORT_CONV_MAX_SEGMENTS} inputs with a weight each expected")
+    _rows2d(out, "out")
+    T = out.shape[0]
+    C = sum(int(x.shape[1]) for x in xs)
+    dt = xs[0].dtype
+    for x, w in zip(xs, ws):
+        _rows2d(x, "x")
+        if x.shape[0] != T or x.dtype != dt or w.dtype != dt or tuple(w.shape) != (x.shape[1], taps) or not w.is_contiguous():
+            raise KernelError(f"short_conv: inputs [T, n] and contiguous weights [n, {taps}] of one dtype expected")
+    if out.dtype != torch.float32 or out.shape[1] != C:
+        raise KernelError(f"short_conv: out must be 32-bit [T, {C}]")
+    if taps > 1 and (state is None or state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (taps - 1, C)
+                     or not state.is_contiguous()):
+        raise KernelError(f"short_conv: state must be contiguous float32 [slots, {taps - 1}, {C}]")
+    _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
+    _i32(ctx.q_start, "q_start", ctx.num_rows)
+    _i32(ctx.state_slots, "state_slots", ctx.num_rows)
+    n = len(xs)
+    ptrs = (ctypes.c_void_p * n)(*[x.data_ptr() for x in xs])
+    wptrs = (ctypes.c_void_p * n)(*[w.data_ptr() for w in ws])
+    strides = (ctypes.c_int * n)(*[x.stride(0) for x in xs])
+    widths = (ctypes.c_int * n)(*[x.shape[1] for x in xs])
+    _check(_lib().ri_short_conv(n, ptrs, strides, wptrs, widths, _dt(xs[0]), int(taps), int(bool(silu)), _ptr(state),
+                                state.shape[0] if state is not None else 1, _ptr(out), out.stride(0), _ptr(ctx.cu_q),
+                                _ptr(ctx.q_start), _ptr(ctx.state_slots), ctx.num_rows, T, int(ctx.max_q_len), _stream()))
+
+
+def gated_delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta_in: torch.Tensor, decay_in: torch.Tensor,
+                     A: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor, out: torch.Tensor, ctx,
+                     H: int, Hk: int, dk: int, dv: int, unit_eps: float = 1e-6, q_scale: float = 1.0) -> None:
+    """Walk each request's tokens of the step through ``state[slot] [H, dk, dv]`` (32-bit) by the gated
+    delta rule: ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q`` with
+    ``beta = sigmoid(beta_in)``, ``g = exp(-A softplus(decay_in + dt_bias))`` (one a head and token), q and k
+    divided by ``sqrt(|.|^2 + unit_eps)`` and q times ``q_scale``.  ``q, k [T, Hk dk]``, ``v [T, H dv]`` 32-bit
+    (columns allowed); head h reads q/k head ``h // (H // Hk)``; ``beta_in, decay_in [T, H]`` activations;
+    ``A, dt_bias [H]`` 32-bit; ``out [T, H dv]`` 32-bit.  A request's first tokens start from zeros."""
+    _dev(q, k, v, beta_in, decay_in, A, dt_bias, state, out)
+    for t, name in ((q, "q"), (k, "k"), (v, "v"), (out, "out"), (beta_in, "beta_in"), (decay_in, "decay_in")):
+        _rows2d(t, name)
+    T = q.shape[0]
+    if tuple(q.shape) != (T, Hk * dk) or tuple(k.shape) != (T, Hk * dk) or tuple(v.shape) != (T, H * dv) \
+            or tuple(out.shape) != (T, H * dv) or any(t.dtype != torch.float32 for t in (q, k, v, out)):
+        raise KernelError("gated_delta_scan: 32-bit q, k [T, Hk dk], v [T, H dv] and out [T, H dv] expected")
+    if tuple(beta_in.shape) != (T, H) or tuple(decay_in.shape) != (T, H) or beta_in.dtype != decay_in.dtype:
+        raise KernelError("gated_delta_scan: beta_in and decay_in must be [T, H] of one dtype")
+    if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (H, dk, dv) or not state.is_contiguous():
+        raise KernelError(f"gated_delta_scan: state must be contiguous float32 [slots, {H}, {dk}, {dv}]")
+    _f32_vec(A, H, "gated_delta_scan: A")
+    _f32_vec(dt_bias, H, "gated_delta_scan: dt_bias")
+    _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
+    _i32(ctx.q_start, "q_start", ctx.num_rows)
+    _i32(ctx.state_slots, "state_slots", ctx.num_rows)
+    _check(_lib().ri_gated_delta_scan(
+        _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(beta_in), beta_in.stride(0),
+        _ptr(decay_in), decay_in.stride(0), _dt(beta_in), _ptr(A), _ptr(dt_bias), ctypes.c_float(unit_eps),
+        ctypes.c_float(q_scale), _ptr(state), state.shape[0], _ptr(out), out.stride(0), _ptr(ctx.cu_q), _ptr(ctx.q_start),
+        _ptr(ctx.state_slots), ctx.num_rows, T, H, Hk, dk, dv, _stream()))

@@ -25,6 +25,10 @@ class LayerCall:
     layer: int                   # index into DecoderModel.layers
     cache: Optional[int] = None  # cache id; None = this call's own position in the run order
     write: bool = True           # False: read the cache, do not write it
+    # (index into DecoderModel.stream_parts, argument): that part acts on the residual stream right
+    # before this call, ``part.forward(ctx, x, embedded, argument)`` with ``embedded`` the rows as the
+    # embedding left them (a stretch of layers that runs again starts each pass this way)
+    enter: Optional[tuple] = None
 
 
 class DecoderModel(Part):
@@ -32,8 +36,10 @@ class DecoderModel(Part):
                  final_norm, lm_head: LMHead,
                  position_encodings: Sequence[PositionEncoding] = (),
                  schedule: Optional[Sequence[LayerCall]] = None,
-                 names: Optional[Dict[str, str]] = None):
+                 names: Optional[Dict[str, str]] = None, stream_parts: Sequence = ()):
+        """``stream_parts``: ``[(tensor name prefix, part)]`` that ``LayerCall.enter`` refers to."""
         self.config = config
+        self.stream_parts = list(stream_parts)
         self.embed = embed
         self.layers = list(layers)
         self.final_norm = final_norm
@@ -42,8 +48,9 @@ class DecoderModel(Part):
         if schedule is None:
             schedule = [LayerCall(i) for i in range(len(self.layers))]
         self.schedule: List[LayerCall] = [
-            LayerCall(c.layer, c.cache if c.cache is not None else pos, c.write)
+            LayerCall(c.layer, c.cache if c.cache is not None else pos, c.write, c.enter)
             for pos, c in enumerate(schedule)]
+        self.keeps_embedded = any(c.enter is not None for c in self.schedule)
         for c in self.schedule:
             if not (0 <= c.layer < len(self.layers)):
                 raise ValueError(f"run order names layer {c.layer}, the model has {len(self.layers)}")
@@ -61,6 +68,8 @@ class DecoderModel(Part):
             yield self.names["layer"].format(i=i), layer
         yield self.names["final_norm"], self.final_norm
         yield self.names["lm_head"], self.lm_head
+        for prefix, part in self.stream_parts:
+            yield prefix, part
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         specs: Dict[str, ParamSpec] = {}
@@ -108,6 +117,13 @@ class DecoderModel(Part):
         for pe in self.position_encodings:
             pe.on_embedding(ctx, x)
         hidden = Hidden(x)
+        embedded = None
+        if self.keeps_embedded:
+            # the rows as the embedding left them, for the parts that add them again later
+            embedded = ws.get("model.embedded", T, self.hidden_size, torch.float32)
+            self.embed.forward(ctx, ctx.token_ids, embedded)
+            for pe in self.position_encodings:
+                pe.on_embedding(ctx, embedded)
         W = ctx.num_want
         # Only the rows whose logits are wanted matter after the last block's mixer: a long prompt
         # portion that wants one row (or none) runs that block's feed-forward on that row alone.
@@ -120,9 +136,16 @@ class DecoderModel(Part):
         for n, call in enumerate(self.schedule):
             cache = caches.view(call.cache, call.write) if call.cache in caches else None
             layer = self.layers[call.layer]
+            if call.enter is not None:
+                if hidden.pending is not None or hidden.deferred is not None:
+                    raise RuntimeError("a part that acts on the stream between two layers needs the stream complete")
+                self.stream_parts[call.enter[0]][1].forward(ctx, hidden.x, embedded, call.enter[1])
+                hidden.act = None
             if n + 1 < len(self.schedule):
                 nxt = self.layers[self.schedule[n + 1].layer]
                 follow = nxt.entry() if hasattr(nxt, "entry") else None
+                if self.schedule[n + 1].enter is not None:
+                    follow = None                    # the stream changes before the next layer reads it
             else:
                 follow = (self.final_norm, self.lm_head) if all_rows else None
             kw = {"follow": follow} if follow is not None and getattr(layer, "takes_follow", False) else {}

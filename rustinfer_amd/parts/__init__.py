@@ -1,13 +1,13 @@
 from .base import (FeedForward, Mixer, Norm, PagedKVNeed, ParamSpec, Part, PositionEncoding,
                    ProjectedPart, ProjectionSet, Runtime, StateNeed, stored_to)
-from .norm import OutputRMSNorm, RMSNorm
+from .norm import LayerNorm, OutputRMSNorm, RMSNorm
 from .rope import RotaryEmbedding, rotary_frequencies
 from .linear import Linear
 from .embed import Embedding, LMHead
-from .mlp import DenseMLP, MoEFeedForward, SwiGLUMLP
+from .mlp import DenseMLP, MoEFeedForward, PolyNormMLP, SwiGLUMLP
 from .attention import LatentAttention, PagedAttention, WindowAttention
-from .recurrent import GeneralDeltaRule, LightningAttention, Retention
-from .block import Hidden, ParallelBlock, PostNormBlock, PreNormBlock
+from .recurrent import GatedDeltaRule, GeneralDeltaRule, LightningAttention, Retention
+from .block import Hidden, ParallelBlock, PostNormBlock, PreNormBlock, SandwichBlock
 from .registry import (MIXERS, FEED_FORWARDS, NORMS, POSITION_ENCODINGS, register_mixer,
                        register_feed_forward, register_norm, register_position_encoding,
                        make_part)

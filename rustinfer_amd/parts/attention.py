@@ -267,19 +267,25 @@ class LatentAttention(ProjectedPart, Mixer):
     checkpoint pairs feature 2i with 2i + 1, so the rows that make the rotated parts are reordered
     when they are loaded (even features, then odd ones), which leaves every score as it was.  More than 32 heads run as several calls of the
     attention kernels over the same cache.
-    Tensor names: ``q, dkv, dkv.norm, uk, uv, o`` unless given."""
+    ``window``: a position sees itself and the ``window - 1`` before it (None: all); the cache gives back the
+    pages the window has passed.  ``sink``: a learned number a head (tensor ``sink``) whose exponential joins
+    the softmax's denominator; it has no key and no value and is not scaled.
+    Tensor names: ``q, dkv, dkv.norm, uk, uv, o, sink`` unless given."""
 
     is_mixer = True
 
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, v_head_dim: int, latent_dim: int,
                  scale: float, norm_eps: float, pos_enc: Optional[PositionEncoding] = None, interleaved: bool = True,
-                 names: Optional[Dict[str, str]] = None):
+                 names: Optional[Dict[str, str]] = None, window: Optional[int] = None, sink: bool = False):
         self.hidden_size = int(hidden_size)
+        self.window = int(window) if window else None
+        self.has_sink = bool(sink)
+        self.sink = None
         self.num_heads, self.head_dim, self.rot_dim = int(num_heads), int(head_dim), int(rot_dim)
         self.v_head_dim, self.latent_dim = int(v_head_dim), int(latent_dim)
         self.scale, self.norm_eps = float(scale), float(norm_eps)
         self.pos_enc, self.interleaved = pos_enc, bool(interleaved)
-        self.names = {"q": "q", "down": "dkv", "norm": "dkv.norm", "uk": "uk", "uv": "uv", "o": "o"}
+        self.names = {"q": "q", "down": "dkv", "norm": "dkv.norm", "uk": "uk", "uv": "uv", "o": "o", "sink": "sink"}
         if names:
             self.names.update(names)
 
@@ -292,11 +298,14 @@ class LatentAttention(ProjectedPart, Mixer):
 
     def own_specs(self):
         n, H, R = self.names, self.num_heads, self.latent_dim
-        return {n["norm"]: ParamSpec((R,), "norm"), n["uk"]: ParamSpec((H * self.head_dim, R)),
-                n["uv"]: ParamSpec((H * self.v_head_dim, R))}
+        specs = {n["norm"]: ParamSpec((R,), "norm"), n["uk"]: ParamSpec((H * self.head_dim, R)),
+                 n["uv"]: ParamSpec((H * self.v_head_dim, R))}
+        if self.has_sink:
+            specs[n["sink"]] = ParamSpec((H,), mean=0.0, std=1.0)
+        return specs
 
     def cache_need(self):
-        return PagedKVNeed(1, self.latent_dim + self.rot_dim, None, self.latent_dim)
+        return PagedKVNeed(1, self.latent_dim + self.rot_dim, self.window, self.latent_dim)
 
     def _pairs_apart(self, part: torch.Tensor) -> torch.Tensor:
         """Rows of one rotated part [rot_dim, hidden] with the turned pairs' halves apart."""
@@ -326,6 +335,8 @@ class LatentAttention(ProjectedPart, Mixer):
         uk = tensors[n["uk"]].to(device=rt.device, dtype=rt.dtype)
         self.w_absorb = uk.view(H, self.head_dim, R).transpose(1, 2).contiguous()        # [H, R, head_dim]: W_uk,h^T
         self.w_value = tensors[n["uv"]].to(device=rt.device, dtype=rt.dtype).contiguous().view(H, self.v_head_dim, R)
+        if self.has_sink:
+            self.sink = tensors[n["sink"]].to(device=rt.device, dtype=torch.float32).contiguous()
 
     def core(self, ctx, proj, act, cache) -> None:
         ops, n, ws = self.rt.ops, self.names, ctx.workspace
@@ -342,5 +353,6 @@ class LatentAttention(ProjectedPart, Mixer):
         for h0 in range(0, H, self.heads_a_call):
             n = min(self.heads_a_call, H - h0)
             ops.window_attention(q_lat[:, h0 * (R + r):(h0 + n) * (R + r)], lat[:, h0 * R:(h0 + n) * R], n, 1, R + r, R,
-                                 cache.k, cache.v, table, cache.page_size, ctx, self.scale, 0, None, False)
+                                 cache.k, cache.v, table, cache.page_size, ctx, self.scale, self.window or 0, None, False,
+                                 sink=self.sink[h0:h0 + n] if self.sink is not None else None)
         ops.head_linear(lat, R, self.w_value, act, self.v_head_dim)

@@ -79,9 +79,16 @@ class PagedKVNeed:
 
 @dataclass(frozen=True)
 class StateNeed:
-    """A fixed-size state for each live request, ``shape`` elements of ``dtype``."""
+    """A fixed-size state for each live request, ``shape`` elements of ``dtype``.  ``extra``: further
+    tensors of the same request's slot, ``((name, shape, dtype), ...)`` (the last inputs of a short
+    convolution beside a state matrix, say); the mixer finds them in ``StateView.extra[name]``."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    extra: Tuple[Tuple[str, Tuple[int, ...], torch.dtype], ...] = ()
+
+    def all_tensors(self):
+        """[(name, shape, dtype)] of every tensor a slot holds; the main one is called ``""``."""
+        return [("", tuple(self.shape), self.dtype)] + [(n, tuple(s), d) for n, s, d in self.extra]
 
 
 @dataclass
@@ -337,12 +344,18 @@ class ProjectionSet:
     starts at a multiple of eight columns (16 bytes in bfloat16), the gaps being rows and columns
     of zeros."""
 
-    def __init__(self, hidden_size: int, members):
+    def __init__(self, hidden_size: int, members, extra_in=()):
+        """``extra_in``: ``[(tensor name, rows)]`` of further projections of the same input that belong to
+        whoever owns the set (a gate on a sub-layer's result, say); their columns are ``extra_views``."""
         from .linear import Linear
         self.hidden_size = int(hidden_size)
         self.members = list(members)                     # [(prefix, part)]
         self.in_slices, self.act_slices = [], []
         n_in = n_act = 0
+        self.extra_slices = {}
+        for name, rows in extra_in:
+            self.extra_slices[name] = (n_in, int(rows))
+            n_in = _up8(n_in + int(rows))
         for _, part in self.members:
             views = {}
             for name, rows in part.in_projections():
@@ -366,11 +379,15 @@ class ProjectionSet:
             specs[join_name(prefix, name)] = ParamSpec((self.hidden_size, int(cols)))
             for name, spec in part.own_specs().items():
                 specs[join_name(prefix, name)] = spec
+        for name, (_, rows) in self.extra_slices.items():
+            specs[name] = ParamSpec((rows, self.hidden_size))
         return specs
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         w_in = torch.zeros((self.n_in, self.hidden_size), device=rt.device, dtype=rt.dtype)
+        for name, (c0, rows) in self.extra_slices.items():
+            w_in[c0:c0 + rows] = tensors[name].to(device=rt.device, dtype=rt.dtype)
         w_out = torch.zeros((self.hidden_size, self.n_act), device=rt.device, dtype=rt.dtype)
         self._gaps, end = [], 0
         for (prefix, part), views, (a0, cols) in zip(self.members, self.in_slices, self.act_slices):
@@ -399,6 +416,9 @@ class ProjectionSet:
 
     def views(self, i: int, proj):
         return {name: proj[:, c0:c0 + rows] for name, (c0, rows) in self.in_slices[i].items()}
+
+    def extra_views(self, proj):
+        return {name: proj[:, c0:c0 + rows] for name, (c0, rows) in self.extra_slices.items()}
 
     def act_view(self, i: int, act):
         a0, cols = self.act_slices[i]

@@ -283,3 +283,137 @@ class PostNormBlock(Part):
         if self.ffn is not None:
             self.ffn_norm.add(ctx, x, self.ffn.forward(ctx, inp), act)
         hidden.act = act
+
+
+class SandwichBlock(Part):
+    """A norm before and after each sub-layer, and a gate on what the sub-layer returns:
+    ``h = norm1(x); x <- x + norm1b(mixer(h) * sigmoid(W_g1 h + b_g1))``, then the same around the
+    feed-forward with ``norm2``, ``norm2b`` and ``W_g2``.  The norms are ``LayerNorm``; the feed-forward
+    may be absent.
+
+    The gate reads what its sub-layer reads, so with a ``ProjectedPart`` its matrix is stacked on the
+    part's in-projections (one product); any other sub-layer gets a product for the gate beside it.
+    Gate, output norm and residual add are one kernel, which also leaves the input of the sub-layer that
+    comes next where that sub-layer's norm is a ``LayerNorm`` (the norm's own kernel then runs only at a
+    block's start where something else changes the stream first).  A sub-layer may have
+    ``out_bias`` (32-bit, the model's width): it is added to what the sub-layer returns."""
+
+    takes_follow = True
+
+    def __init__(self, hidden_size: int, mixer_norm: Norm, mixer: Mixer, mixer_out_norm: Norm,
+                 ffn_norm: Optional[Norm] = None, ffn: Optional[FeedForward] = None, ffn_out_norm: Optional[Norm] = None,
+                 names: Optional[Dict[str, str]] = None):
+        if mixer is None or mixer_norm is None or mixer_out_norm is None:
+            raise ValueError("a block needs a mixer with a norm before and after it")
+        if len({ffn is None, ffn_norm is None, ffn_out_norm is None}) != 1:
+            raise ValueError("a feed-forward and its two norms come together")
+        self.hidden_size = int(hidden_size)
+        self.mixer_norm, self.mixer, self.mixer_out_norm = mixer_norm, mixer, mixer_out_norm
+        self.ffn_norm, self.ffn, self.ffn_out_norm = ffn_norm, ffn, ffn_out_norm
+        self.names = {"mixer_norm": "norm1", "mixer": "mix", "mixer_out_norm": "norm1b", "mixer_gate": "rg1",
+                      "ffn_norm": "norm2", "ffn": "mlp", "ffn_out_norm": "norm2b", "ffn_gate": "rg2", "gate_bias": "b"}
+        if names:
+            self.names.update(names)
+        self.halves = [self._half("mixer", mixer)] + ([self._half("ffn", ffn)] if ffn is not None else [])
+
+    def _half(self, key: str, part):
+        from .base import ProjectedPart
+        from .linear import Linear
+        gate = self.names[key + "_gate"]
+        half = {"key": key, "part": part, "gate": gate, "norm": getattr(self, key + "_norm"),
+                "out_norm": getattr(self, key + "_out_norm"), "set": None, "gate_linear": None, "gate_bias": None}
+        if isinstance(part, ProjectedPart):
+            half["set"] = ProjectionSet(self.hidden_size, [(self.names[key], part)], extra_in=[(gate, self.hidden_size)])
+        else:
+            half["gate_linear"] = Linear(self.hidden_size, self.hidden_size)
+        return half
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        specs = {}
+        for half in self.halves:
+            key = half["key"]
+            for which in ("norm", "out_norm"):
+                prefix = self.names[key + "_" + which]
+                for name, spec in half[which].param_specs().items():
+                    specs[join_name(prefix, name)] = spec
+            if half["set"] is not None:
+                specs.update(half["set"].param_specs())
+            else:
+                for name, spec in half["part"].param_specs().items():
+                    specs[join_name(self.names[key], name)] = spec
+                specs[half["gate"]] = ParamSpec((self.hidden_size, self.hidden_size))
+            specs[join_name(half["gate"], self.names["gate_bias"])] = ParamSpec((self.hidden_size,), mean=0.0, std=0.5)
+        return specs
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        for half in self.halves:
+            key = half["key"]
+            for which in ("norm", "out_norm"):
+                half[which].load(narrow_tensors(tensors, self.names[key + "_" + which]), rt)
+            if half["set"] is not None:
+                half["set"].load(tensors, rt)
+                half["part"].rt = rt
+            else:
+                half["part"].load(narrow_tensors(tensors, self.names[key]), rt)
+                half["gate_linear"].set_weight(tensors[half["gate"]], rt)
+            half["gate_bias"] = tensors[join_name(half["gate"], self.names["gate_bias"])].to(
+                device=rt.device, dtype=torch.float32).contiguous()
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", True) for h in self.halves for p in (h["part"], h["norm"], h["out_norm"]))
+
+    def can_cut_rows(self) -> bool:
+        return False
+
+    def entry(self):
+        return (self.mixer_norm, self.mixer)
+
+    def _run_half(self, ctx, hidden: Hidden, half, cache, after, only_state: bool = False) -> None:
+        """One sub-layer with its gate, output norm and residual add; ``after``: the (norm, sub-layer) that
+        come next, whose input is made in the same pass if that norm allows it."""
+        ops, ws = self.rt.ops, ctx.workspace
+        x, T = hidden.x, hidden.x.shape[0]
+        which = "a" if half["key"] == "mixer" else "b"       # two buffers: one is read while the other is filled
+        inp = hidden.input_behind(ctx, half["norm"], ws.get("block.normed." + which, T, self.hidden_size, self.rt.dtype))
+        part = half["part"]
+        if half["set"] is not None:
+            s = half["set"]
+            proj, act = s.project(ctx, inp)
+            part.core(ctx, s.views(0, proj), s.act_view(0, act), cache)
+            if only_state:
+                return
+            delta, gate = s.output(ctx, act), s.extra_views(proj)[half["gate"]]
+        else:
+            delta = part.forward(ctx, inp, cache) if half["key"] == "mixer" else part.forward(ctx, inp)
+            if only_state:
+                return
+            gate = ws.get("block.gate", T, self.hidden_size, self.rt.dtype)
+            half["gate_linear"].forward(inp, gate)
+        next_norm = next_out = None
+        if after is not None and getattr(after[0], "layer_norm", False) and after[0].dim == self.hidden_size \
+                and after[0].eps == half["out_norm"].eps:
+            other = "b" if which == "a" else "a"
+            next_norm = (after[0].weight, after[0].bias)
+            next_out = ws.get("block.normed." + other, T, self.hidden_size, self.rt.dtype)
+        out_norm = half["out_norm"]
+        ops.gated_norm_residual(x, delta, out_norm.weight, out_norm.bias, out_norm.eps, gate=gate, gate_bias=half["gate_bias"],
+                                delta_bias=getattr(part, "out_bias", None), next_norm=next_norm, next_out=next_out)
+        hidden.pending, hidden.deferred = None, ((after[0], next_out) if next_out is not None else None)
+
+    def forward(self, ctx, hidden: Hidden, cache, out_rows=None, follow=None) -> None:
+        if hidden.pending is not None:
+            raise RuntimeError("a block whose norms add to the stream themselves needs the stream complete")
+        for i, half in enumerate(self.halves):
+            nxt = self.halves[i + 1] if i + 1 < len(self.halves) else None
+            after = (nxt["norm"], nxt["part"]) if nxt is not None else follow
+            self._run_half(ctx, hidden, half, cache if half["key"] == "mixer" else None, after)
+
+    def update_cache_only(self, ctx, hidden: Hidden, cache) -> None:
+        """The last block of a step whose logits nobody wants: the mixer alone runs, for what it leaves in
+        its cache or state; ``hidden`` is not meaningful afterwards."""
+        self._run_half(ctx, hidden, self.halves[0], cache, None, only_state=True)

@@ -73,3 +73,32 @@ class OutputRMSNorm(Norm):
         """``x`` (32-bit stream) gains the normed ``delta`` ([T, d], or a stack of 32-bit partial sums);
         ``act`` takes the new rows in its dtype, for the sub-layer that reads the stream next."""
         self.rt.ops.norm_residual(x, delta, self.weight, self.eps, mult=self.mult, one_plus=self.one_plus, act=act)
+
+
+class LayerNorm(Norm):
+    """``(x - mean) / sqrt(var + eps) * w + b`` over each row, the variance being the mean of the squared
+    deviations; 32-bit arithmetic, weight and bias kept in 32-bit.  Tensors: the weight under
+    ``weight_name`` ("" where it carries the norm's own name), the bias under that name + ``bias_suffix``."""
+
+    cuts_rows = False
+    plain_rms = False
+    layer_norm = True          # a block may make this norm's output in the pass that last changes the stream
+
+    def __init__(self, dim: int, eps: float, weight_name: str = "weight", bias_name: str = "bias"):
+        self.dim, self.eps = int(dim), float(eps)
+        self.weight_name, self.bias_name = weight_name, bias_name
+        self.weight = self.bias = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {self.weight_name: ParamSpec((self.dim,), "norm"), self.bias_name: ParamSpec((self.dim,), mean=0.0, std=0.1)}
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        f32 = lambda name: tensors[name].to(device=rt.device, dtype=torch.float32).contiguous()
+        self.weight, self.bias = f32(self.weight_name), f32(self.bias_name)
+
+    def forward(self, ctx, x, delta, out, rows=None, x_rows=None):
+        if delta is not None or x_rows is not None:
+            raise RuntimeError("LayerNorm norms a complete stream: nothing pending, no cut to rows")
+        self.rt.ops.layer_norm(x, self.weight, self.bias, self.eps, out, rows)
+        return out

@@ -13,6 +13,11 @@ request's state slot, zeros before its first token):
                          terms read the old state); each head's output is divided by its own root
                          mean square, then a learned weight, the gate and the projection.
 
+``GatedDeltaRule``       ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` with one decay ``g`` and one
+                         write strength ``beta`` a head and token; q, k, v pass a short causal convolution
+                         and silu first, q and k are made unit vectors; each head's output is divided by its
+                         root mean square, times a weight, times ``silu(W_g x)``.
+
 The walk is one kernel for prompt portions and single tokens alike (``csrc/recurrent.hip``);
 everything between the projections and the gated norm's output is 32-bit.
 """
@@ -167,3 +172,91 @@ class Retention(ProjectedPart, Mixer):
                         self.v_head_dim, decay=self.decay, rotary=self.pos_enc.rotary() if self.pos_enc is not None else None,
                         k_scale=self.key_scale)
         ops.gated_group_norm(o, None, proj[n["g"]], act, self.v_head_dim, self.norm_eps, gate_activation="silu")
+
+
+class GatedDeltaRule(ProjectedPart, Mixer):
+    """The gated delta rule.  ``q = W_q x`` and ``k = W_k x`` have ``num_kv_heads`` heads of ``head_dim``,
+    ``v = W_v x`` has ``num_heads`` heads of ``v_head_dim``; head h reads q/k head ``h // (num_heads //
+    num_kv_heads)``.  Each of q, k, v passes a causal convolution over time of ``conv_taps`` taps, channel by
+    channel (tensors ``<name>.conv`` ``[channels, taps]``, the last column the current token's, no bias), then
+    silu.  q and k are divided by ``sqrt(|.|^2 + unit_eps)`` head by head, q also times ``q_scale``
+    (``head_dim^(-1/2)`` unless given).  ``beta = sigmoid(W_b x)`` and
+    ``g = exp(-exp(A_log) softplus(W_a x + dt_bias))``, one a head.  Per head, in this order:
+    ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q``.  Each head's ``o`` is divided by its root
+    mean square over ``v_head_dim`` (``norm_eps``), times the weight ``norm`` (``v_head_dim`` entries shared by
+    the heads), times ``silu(W_g x)``; then ``W_o``.
+
+    A request's slot holds the 32-bit state ``[heads, head_dim, v_head_dim]`` and the convolutions' last
+    ``conv_taps - 1`` inputs; everything between the projections and the gated norm's output is 32-bit.
+    Tensor names: ``q, k, v, g, b, a, o, q.conv, k.conv, v.conv, A_log, dt_bias, norm`` unless given."""
+
+    is_mixer = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
+                 conv_taps: int, norm_eps: float, unit_eps: float = 1e-6, q_scale: Optional[float] = None,
+                 names: Optional[Dict[str, str]] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
+        if conv_taps < 1:
+            raise ValueError("a convolution has one tap at least")
+        self.hidden_size = int(hidden_size)
+        self.num_heads, self.num_kv_heads = int(num_heads), int(num_kv_heads)
+        self.head_dim, self.v_head_dim, self.conv_taps = int(head_dim), int(v_head_dim), int(conv_taps)
+        self.norm_eps, self.unit_eps = float(norm_eps), float(unit_eps)
+        self.q_scale = float(q_scale) if q_scale is not None else self.head_dim ** -0.5
+        self.names = {"q": "q", "k": "k", "v": "v", "g": "g", "b": "b", "a": "a", "o": "o", "conv": "conv",
+                      "A_log": "A_log", "dt_bias": "dt_bias", "norm": "norm"}
+        if names:
+            self.names.update(names)
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.num_kv_heads * self.head_dim + self.num_heads * self.v_head_dim
+
+    def in_projections(self):
+        n, ck, cv, H = self.names, self.num_kv_heads * self.head_dim, self.num_heads * self.v_head_dim, self.num_heads
+        return [(n["q"], ck), (n["k"], ck), (n["v"], cv), (n["g"], cv), (n["b"], H), (n["a"], H)]
+
+    def out_projection(self):
+        return (self.names["o"], self.num_heads * self.v_head_dim)
+
+    def own_specs(self):
+        n, ck, cv, H, t = self.names, self.num_kv_heads * self.head_dim, self.num_heads * self.v_head_dim, self.num_heads, self.conv_taps
+        conv = lambda rows: ParamSpec((rows, t), mean=0.0, std=0.5)
+        return {join_conv(n["q"], n["conv"]): conv(ck), join_conv(n["k"], n["conv"]): conv(ck), join_conv(n["v"], n["conv"]): conv(cv),
+                n["A_log"]: ParamSpec((H,), mean=-1.0, std=1.0), n["dt_bias"]: ParamSpec((H,), mean=0.0, std=1.0),
+                n["norm"]: ParamSpec((self.v_head_dim,), "norm")}
+
+    def cache_need(self):
+        extra = ()
+        if self.conv_taps > 1:
+            extra = (("conv", (self.conv_taps - 1, self.conv_channels), torch.float32),)
+        return StateNeed((self.num_heads, self.head_dim, self.v_head_dim), torch.float32, extra)
+
+    def load_own(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        n = self.names
+        if self.conv_taps > rt.ops.SHORT_CONV_MAX_TAPS:
+            raise ValueError(f"a convolution of {self.conv_taps} taps is beyond the kernel ({rt.ops.SHORT_CONV_MAX_TAPS})")
+        f32 = lambda name: tensors[name].to(device=rt.device, dtype=torch.float32).contiguous()
+        self.conv_weights = [tensors[join_conv(n[x], n["conv"])].to(device=rt.device, dtype=rt.dtype).contiguous() for x in ("q", "k", "v")]
+        self.decay_rate = torch.exp(f32(n["A_log"]))                       # A of g = exp(-A softplus(.)), 32-bit
+        self.dt_bias = f32(n["dt_bias"])
+        self.norm_weight = f32(n["norm"]).repeat(self.num_heads)          # the same weight for every head
+
+    def core(self, ctx, proj, act, cache) -> None:
+        ops, n, ws = self.rt.ops, self.names, ctx.workspace
+        T, H, Hk, dk, dv = act.shape[0], self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim
+        ck = Hk * dk
+        mixed = ws.get("gdelta.conv", T, self.conv_channels, torch.float32)
+        ops.short_conv([proj[n["q"]], proj[n["k"]], proj[n["v"]]], self.conv_weights,
+                       cache.extra["conv"] if self.conv_taps > 1 else None, mixed, ctx, self.conv_taps, silu=True)
+        o = ws.get("scan.o", T, H * dv, torch.float32)
+        ops.gated_delta_scan(mixed[:, :ck], mixed[:, ck:2 * ck], mixed[:, 2 * ck:], proj[n["b"]], proj[n["a"]],
+                             self.decay_rate, self.dt_bias, cache.state, o, ctx, H, Hk, dk, dv,
+                             unit_eps=self.unit_eps, q_scale=self.q_scale)
+        ops.gated_group_norm(o, self.norm_weight, proj[n["g"]], act, dv, self.norm_eps, gate_activation="silu")
+
+
+def join_conv(name: str, suffix: str) -> str:
+    return f"{name}.{suffix}"

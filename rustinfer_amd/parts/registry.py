@@ -5,16 +5,16 @@ from __future__ import annotations
 from typing import Callable, Dict
 
 from .attention import LatentAttention, PagedAttention, WindowAttention
-from .mlp import DenseMLP, MoEFeedForward, SwiGLUMLP
-from .norm import OutputRMSNorm, RMSNorm
-from .recurrent import GeneralDeltaRule, LightningAttention, Retention
+from .mlp import DenseMLP, MoEFeedForward, PolyNormMLP, SwiGLUMLP
+from .norm import LayerNorm, OutputRMSNorm, RMSNorm
+from .recurrent import GatedDeltaRule, GeneralDeltaRule, LightningAttention, Retention
 from .rope import RotaryEmbedding
 
 MIXERS: Dict[str, Callable] = {"attention": PagedAttention, "window_attention": WindowAttention,
                                "lightning": LightningAttention, "general_delta": GeneralDeltaRule,
-                               "latent_attention": LatentAttention, "retention": Retention}
-FEED_FORWARDS: Dict[str, Callable] = {"swiglu": SwiGLUMLP, "dense": DenseMLP, "moe": MoEFeedForward}
-NORMS: Dict[str, Callable] = {"rmsnorm": RMSNorm, "output_rmsnorm": OutputRMSNorm}
+                               "latent_attention": LatentAttention, "retention": Retention, "gated_delta": GatedDeltaRule}
+FEED_FORWARDS: Dict[str, Callable] = {"swiglu": SwiGLUMLP, "dense": DenseMLP, "moe": MoEFeedForward, "poly_norm": PolyNormMLP}
+NORMS: Dict[str, Callable] = {"rmsnorm": RMSNorm, "output_rmsnorm": OutputRMSNorm, "layernorm": LayerNorm}
 POSITION_ENCODINGS: Dict[str, Callable] = {"rope": RotaryEmbedding}
 
 _TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
