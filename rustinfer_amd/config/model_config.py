@@ -863,13 +863,10 @@ class PilavikConfig(ModelConfig):
     layers: tuple = ()
     loop_start: int = 0
     loop_stop: int = 0
-    loop_times: int = 1          # 1 with loop_start == loop_stop: no loop
+    loop_times: int = 1
+    has_loop: bool = False       # config.json has a 'loop' (the checkpoint then has the passes' vectors)
     eos_token_ids: tuple = ()
     architecture: str = "Pilavik"
-
-    @property
-    def has_loop(self) -> bool:
-        return self.loop_stop > self.loop_start
 
     @classmethod
     def from_dict(cls, d: Dict[str, Any], where: str = "config.json") -> "PilavikConfig":
@@ -903,7 +900,8 @@ class PilavikConfig(ModelConfig):
         eos_ids = () if eos is None else tuple(_typed(e, "eos_token_id", int, where) for e in (eos if isinstance(eos, list) else [eos]))
         cfg = cls(vocab_size=_require(d, "vocab", int, where), hidden_size=_require(d, "width", int, where),
                   norm_eps=_require(_obj(d, "norm", where), "eps", float, where + ".norm"),
-                  layers=tuple(layers), loop_start=start, loop_stop=stop, loop_times=times, eos_token_ids=eos_ids)
+                  layers=tuple(layers), loop_start=start, loop_stop=stop, loop_times=times, has_loop=loop is not None,
+                  eos_token_ids=eos_ids)
         if cfg.vocab_size <= 0 or cfg.hidden_size <= 0 or not cfg.norm_eps > 0:
             raise ConfigError(f"{where}: vocab and width must be > 0, norm.eps > 0")
         return cfg

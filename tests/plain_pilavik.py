@@ -114,11 +114,16 @@ def gated_expert(h, gate, up, down):
     return (silu(h @ gate.T) * (h @ up.T)) @ down.T
 
 
-def moe_ff(h, p, mlp):
+def moe_ff(h, p, mlp, margins=None):
+    """``margins`` (a list) receives, for every token, by how much the last chosen expert's logit lies
+    above the first one left out."""
     E, top, scale = mlp["router"]["experts"], mlp["router"]["top"], mlp["router"].get("scale", 1.0)
     z = h.to(torch.float64) @ p["router"].to(torch.float64).T
     s = torch.sigmoid(z)
     best = torch.topk(s, top, dim=-1)
+    if margins is not None:
+        ordered = torch.sort(z, dim=-1, descending=True).values
+        margins.append(ordered[:, top - 1] - ordered[:, top] if top < E else torch.full((h.shape[0],), float("inf"), dtype=torch.float64))
     wts = best.values / (best.values.sum(-1, keepdim=True) + 1e-20) * scale
     out = torch.zeros_like(h)
     for e in range(E):
@@ -148,9 +153,9 @@ def sub(tensors, prefix, dtype):
     return {n[len(prefix) + 1:]: t.to(dtype) for n, t in tensors.items() if n.startswith(prefix + ".")}
 
 
-def forward(cfg, tensors, tokens, dtype=torch.float64, keep_layers=False):
+def forward(cfg, tensors, tokens, dtype=torch.float64, keep_layers=False, margins=None):
     """Logits [T, vocab] of one request's tokens; with ``keep_layers`` also the residual stream after
-    every layer run, [runs, T, width]."""
+    every layer run, [runs, T, width].  ``margins``: see ``moe_ff``, one entry for every routed layer run."""
     eps = cfg["norm"]["eps"]
     g = lambda name: tensors[name].to(dtype)
     emb = g("embed")[torch.as_tensor(tokens, dtype=torch.long)]
@@ -178,7 +183,7 @@ def forward(cfg, tensors, tokens, dtype=torch.float64, keep_layers=False):
         if mlp is not None:
             h = layer_norm(x, g(f"{L}.norm2"), g(f"{L}.norm2.b"), eps)
             p = sub(tensors, f"{L}.mlp", dtype)
-            y = poly_norm_ff(h, p, eps) if mlp["kind"] == "dense" else moe_ff(h, p, mlp)
+            y = poly_norm_ff(h, p, eps) if mlp["kind"] == "dense" else moe_ff(h, p, mlp, margins)
             y = y * torch.sigmoid(h @ g(f"{L}.rg2").T + g(f"{L}.rg2.b"))
             x = x + layer_norm(y, g(f"{L}.norm2b"), g(f"{L}.norm2b.b"), eps)
         if keep_layers:
