@@ -476,19 +476,86 @@ class BeloraxBench(TedelixBench):
                 self.scan_flops_per_token += 2.0 * 2 * m.heads * m.dim * m.vdim
 
 
-DESIGNS = {"tedelix": (TedelixBench, "llama", TEDELIX_PATTERN), "belorax": (BeloraxBench, "tedelix", BELORAX_PATTERN)}
+# Pilavik at the layer sizes of the Llama shapes: the same width, heads and number of layer RUNS: the
+# list is two layers shorter and its layers 2 and 3 run twice; two layers of the gated delta rule
+# (key heads as the shape's key/value heads, convolutions of four taps) then one of latent attention
+# (Belorax's latent and rotated part, a window of 1,024 keys, a sink); feed-forwards that norm powers
+# alternate with eight experts of a quarter of their width, two a token, and a shared one of that width.
+PILAVIK_PATTERN = ("delta", "delta", "latent_attention")
+
+
+def pilavik_config(shape_name, layers=0, window=1024):
+    s = SHAPES[shape_name]
+    H, G, hd, W, ff = s["num_attention_heads"], s["num_key_value_heads"], s["head_dim"], s["hidden_size"], s["intermediate_size"]
+    runs = layers or s["num_hidden_layers"]
+    loop = dict(start=2, stop=4, times=2) if runs >= 6 else None
+    out = []
+    for i in range(runs - 2 if loop else runs):
+        kind = PILAVIK_PATTERN[i % len(PILAVIK_PATTERN)]
+        if kind == "delta":
+            mixer = dict(heads=H, kv_heads=G, dim=hd, vdim=hd, conv=4)
+        else:
+            r = hd // 2
+            mixer = dict(heads=H, dim=hd, rot_dim=r, vdim=hd, kv_rank=256 - r, scale=(hd + r) ** -0.5,
+                         rot=dict(base=10000.0, dims=r), mask=dict(size=window))
+        mlp = dict(kind="dense", ff=ff) if i % 2 == 0 else dict(kind="moe", expert=dict(ff=ff // 4), shared=dict(ff=ff // 4),
+                                                                router=dict(experts=8, top=2, scale=1.5))
+        out.append(dict(type=kind, mixer=mixer, mlp=mlp))
+    conf = dict(architecture="Pilavik", vocab=s["vocab_size"], width=W, norm=dict(eps=1e-5), layers=out)
+    if loop:
+        conf["loop"] = loop
+    return conf
+
+
+class PilavikBench(TedelixBench):
+    """The same measurements on a Pilavik model of a Llama shape's sizes."""
+
+    def design_config(self, shape_name, args):
+        return pilavik_config(shape_name, args.layers, self.window)
+
+    def account(self, cfg, el):
+        # every layer RUN reads its weights and its own cache or state: a layer of the stretch counts `times` times
+        self.window_kv_bytes = self.state_bytes = 0
+        self.attn_flops_per_key = self.scan_flops_per_token = 0
+        again = 0
+        for i, layer in enumerate(cfg.layers):
+            times = cfg.loop_times if cfg.has_loop and cfg.loop_start <= i < cfg.loop_stop else 1
+            m = layer.mixer
+            if layer.type == "latent_attention":
+                self.window_kv_bytes += times * (2 * m.kv_rank + m.rot_dim) * el
+                self.attn_flops_per_key += times * 2.0 * m.heads * (2 * m.kv_rank + m.rot_dim)
+                self.scan_flops_per_token += times * 2.0 * m.heads * m.kv_rank * (m.dim + m.vdim)
+            else:
+                self.state_bytes += times * 2 * 4 * m.heads * m.dim * m.vdim
+                self.scan_flops_per_token += times * 2.0 * 4 * m.heads * m.dim * m.vdim
+            if times > 1:
+                again += (times - 1) * sum(_count(spec.shape) for name, spec in self.engine.model.param_specs().items()
+                                           if name.startswith(f"l{i}."))
+        self.params += again                      # weights read (and multiplied) a step, not weights stored
+        self.weight_bytes = el * self.params
+
+
+def _count(shape):
+    n = 1
+    for d in shape:
+        n *= int(d)
+    return n
+
+
+DESIGNS = {"tedelix": (TedelixBench, "llama", TEDELIX_PATTERN), "belorax": (BeloraxBench, "tedelix", BELORAX_PATTERN),
+           "pilavik": (PilavikBench, "belorax", PILAVIK_PATTERN)}
 
 
 def design_record(args, peaks):
-    """``--design tedelix|belorax``: decode at the main batch and prefill of 2,048 tokens for models of
-    that design at the sizes of ``--design-shapes``, each beside the closest other design at the same
-    sizes (Tedelix beside Llama, Belorax beside Tedelix)."""
+    """``--design tedelix|belorax|pilavik``: decode at the main batch and prefill of 2,048 tokens for models
+    of that design at the sizes of ``--design-shapes``, each beside the closest other design at the same
+    sizes (Tedelix beside Llama, Belorax beside Tedelix, Pilavik beside Belorax)."""
     design_cls, beside, pattern = DESIGNS[args.design]
-    others = {"llama": Bench, "tedelix": TedelixBench}
+    others = {"llama": Bench, "tedelix": TedelixBench, "belorax": BeloraxBench}
     out = {"metric": "decode tok/s at batch %d and prefill tok/s at 2,048 tokens: %s beside %s at equal layer sizes" % (args.batch, args.design, beside),
            "unit": "tok/s", "dtype": args.dtype, "data": "synthetic: random weights, random token ids", "peaks": peaks,
            "pattern": list(pattern), "shapes": {}}
-    if args.design == "tedelix":
+    if args.design in ("tedelix", "pilavik"):
         out["window"] = 1024
     steps = max(MIN_POINT_STEPS, args.steps)
     for name in args.design_shapes.split(","):
@@ -585,11 +652,11 @@ def main() -> int:
                     help="only time the sampling kernels on 1, 8 and 64 rows of the shape's vocabulary")
     ap.add_argument("--no-gemm-tune", action="store_true",
                     help="keep the GEMM library's own choice of kernel for the prompt's products")
-    ap.add_argument("--design", default="llama", choices=["llama", "tedelix", "belorax"],
-                    help="tedelix, belorax: only decode and prefill of models of that design at the sizes of --design-shapes, "
-                         "each beside the closest other design at the same sizes (Tedelix beside Llama, Belorax beside "
-                         "Tedelix; the default workload is not run)")
-    ap.add_argument("--design-shapes", default="1b,3b", help="shapes for --design tedelix|belorax, with commas between them")
+    ap.add_argument("--design", default="llama", choices=["llama", "tedelix", "belorax", "pilavik"],
+                    help="tedelix, belorax, pilavik: only decode and prefill of models of that design at the sizes of "
+                         "--design-shapes, each beside the closest other design at the same sizes (Tedelix beside Llama, "
+                         "Belorax beside Tedelix, Pilavik beside Belorax; the default workload is not run)")
+    ap.add_argument("--design-shapes", default="1b,3b", help="shapes for --design other than llama, with commas between them")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

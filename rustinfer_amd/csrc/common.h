@@ -44,6 +44,35 @@ __device__ __forceinline__ float ld_f32(const bf16_t* p) { return bf16_to_f32(*p
 __device__ __forceinline__ void st_f32(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st_f32(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 
+// VEC values a thread and load (4: 16 bytes of 32-bit floats, 8 of bfloat16), widened to 32-bit.
+template <int VEC> struct VecLoad;
+template <> struct VecLoad<1> {
+    static __device__ __forceinline__ void ld(const float* p, float* v) { v[0] = *p; }
+    static __device__ __forceinline__ void ld(const bf16_t* p, float* v) { v[0] = bf16_to_f32(*p); }
+    static __device__ __forceinline__ void st(float* p, const float* v) { *p = v[0]; }
+    static __device__ __forceinline__ void st(bf16_t* p, const float* v) { *p = f32_to_bf16(v[0]); }
+};
+template <> struct VecLoad<4> {
+    static __device__ __forceinline__ void ld(const float* p, float* v) {
+        const float4 t = *reinterpret_cast<const float4*>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    static __device__ __forceinline__ void ld(const bf16_t* p, float* v) {
+        const uint2 t = *reinterpret_cast<const uint2*>(p);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void st(float* p, const float* v) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+    static __device__ __forceinline__ void st(bf16_t* p, const float* v) {
+        uint2 t;
+        t.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+        t.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+        *reinterpret_cast<uint2*>(p) = t;
+    }
+};
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -66,6 +95,16 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     float r = 0.f;
     for (int i = 0; i < nw; ++i) r += red[i];
     return r;
+}
+// Three sums at once, left in a, b and c for every thread; `red` holds 48 floats.  Two barriers.
+__device__ __forceinline__ void block_sum3(float& a, float& b, float& c, float* red) {
+    a = wave_sum(a); b = wave_sum(b); c = wave_sum(c);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if (lane == 0) { red[wave] = a; red[16 + wave] = b; red[32 + wave] = c; }
+    __syncthreads();
+    a = b = c = 0.f;
+    for (int i = 0; i < nw; ++i) { a += red[i]; b += red[16 + i]; c += red[32 + i]; }
 }
 __device__ __forceinline__ float block_max(float v, float* red) {
     v = wave_max(v);

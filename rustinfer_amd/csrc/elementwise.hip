@@ -53,34 +53,6 @@ extern "C" int ri_embed(const int* ids, const int* device_tokens, const void* ta
 // delta may be a stack of `parts` 32-bit partial sums (what a product split over K leaves).
 // VEC elements per thread and load: 4 when d % 4 == 0, else 1.
 // ---------------------------------------------------------------------------
-template <int VEC> struct VecLoad;
-template <> struct VecLoad<1> {
-    static __device__ __forceinline__ void ld(const float* p, float* v) { v[0] = *p; }
-    static __device__ __forceinline__ void ld(const bf16_t* p, float* v) { v[0] = bf16_to_f32(*p); }
-    static __device__ __forceinline__ void st(float* p, const float* v) { *p = v[0]; }
-    static __device__ __forceinline__ void st(bf16_t* p, const float* v) { *p = f32_to_bf16(v[0]); }
-};
-template <> struct VecLoad<4> {
-    static __device__ __forceinline__ void ld(const float* p, float* v) {
-        const float4 t = *reinterpret_cast<const float4*>(p);
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-    }
-    static __device__ __forceinline__ void ld(const bf16_t* p, float* v) {
-        const uint2 t = *reinterpret_cast<const uint2*>(p);
-        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
-        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
-    }
-    static __device__ __forceinline__ void st(float* p, const float* v) {
-        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
-    }
-    static __device__ __forceinline__ void st(bf16_t* p, const float* v) {
-        uint2 t;
-        t.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
-        t.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
-        *reinterpret_cast<uint2*>(p) = t;
-    }
-};
-
 // PARTS > 0: that many partial sums, all requested before any is added; 0: a runtime count.
 template <typename TD, typename TW, typename TO, int BLOCK, int VEC, int PARTS>
 __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(

@@ -343,11 +343,13 @@ def test_routing_kernels_with_sigmoid_scores_and_a_shared_expert(E, top, F, shar
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("width,parts", [(64, 1), (100, 3), (4096 + 8, 2), (33, 1)])
-def test_layer_norms_and_the_gated_norm_on_a_sublayers_output(dtype, width, parts):
+@pytest.mark.parametrize("width,parts,T", [(64, 1, 9), (100, 3, 9), (4096 + 8, 2, 9), (33, 1, 9), (1024, 8, 3), (2048, 4, 8), (1026, 5, 9),
+                                           (1536, 1, 300), (4608, 2, 260), (16384, 1, 9)])
+def test_layer_norms_and_the_gated_norm_on_a_sublayers_output(dtype, width, parts, T):
+    """Rows short and long, of lengths that do and do not allow loads of four values, few rows (many
+    threads a row) and many, one to eight partial sums."""
     from rustinfer_amd.kernels import ops
     g = torch.Generator().manual_seed(width)
-    T = 9
     act_dtype = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     x = torch.randn(T, width, generator=g) * 3.0 + 1.0
     vecs = [(torch.randn(width, generator=g) * 0.3 + m).to(DEV) for m in (1.0, 0.0, 0.0, 0.1, 1.0, 0.0)]
@@ -366,12 +368,33 @@ def test_layer_norms_and_the_gated_norm_on_a_sublayers_output(dtype, width, part
     tol = 1e-2 if dtype == "bfloat16" else 1e-5
     assert rel(xd.double().cpu().numpy(), new.numpy()) < 1e-5
     assert rel(out.double().cpu().numpy(), nxt.numpy()) < tol
-    rows = torch.tensor([5, 0, 8], dtype=torch.int32, device=DEV)
+    picked = [T - 2, 0, T - 1]
+    rows = torch.tensor(picked, dtype=torch.int32, device=DEV)
     some = torch.empty(3, width, device=DEV, dtype=act_dtype)
     ops.layer_norm(xd, w2, b2, 1e-5, some, rows)
-    assert rel(some.double().cpu().numpy(), nxt[[5, 0, 8]].numpy()) < tol
+    assert rel(some.double().cpu().numpy(), nxt[picked].numpy()) < tol
     ops.stream_add(xd, out, w1)
     assert rel(xd.double().cpu().numpy(), (new + out.double().cpu() + w1.double().cpu()).numpy()) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,T,bias", [(24, 5, True), (1023, 5, True), (8192, 8, True), (20480, 3, False), (4100, 300, True), (6144, 257, False)])
+def test_the_activation_that_norms_powers(dtype, n, T, bias):
+    """Rows that fit a thread's registers and rows that do not, few rows and many, columns of wider buffers."""
+    from rustinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(n + T)
+    dt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    wide = (torch.randn(T, n + 16, generator=g) * 1.5).to(dt)
+    z = wide[:, 8:8 + n].double()
+    b = torch.randn(n, generator=g) * 0.5 if bias else None
+    if bias:
+        z = z + b.double()
+    a_, b_, c_, e_ = 0.7, -0.35, 0.2, 0.05
+    ref = a_ * P.rms(z, 1e-5) + b_ * P.rms(z * z, 1e-5) + c_ * P.rms(z * z * z, 1e-5) + e_
+    out = torch.zeros(T, n + 4, device=DEV, dtype=dt)
+    ops.poly_norm(wide.to(DEV)[:, 8:8 + n], b.to(DEV) if bias else None, (a_, b_, c_, e_), 1e-5, out[:, 4:4 + n])
+    assert rel(out[:, 4:4 + n].double().cpu().numpy(), ref.numpy()) < (1e-2 if dtype == "bfloat16" else 1e-5)
+    assert float(out[:, :4].abs().max()) == 0.0
 
 
 @pytest.mark.parametrize("taps", [1, 2, 4, 8])
