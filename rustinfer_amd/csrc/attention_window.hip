@@ -659,7 +659,12 @@ int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, con
         // beyond eight heads a key/value head, four heads a wave (one pass over the block of keys): a step
         // of few rows then has waves enough to hide the loads of one another (32 heads on one latent, 8 rows
         // of 2,048 keys: 258 us with all heads in one wave, 78 with eight, 47 with four, 74 with two)
-        const int heads_a_wave = G <= 8 ? G : 4, stretches = (G + heads_a_wave - 1) / heads_a_wave;
+        // (a window of 1,024 keys leaves half as many waves as 2,048 keys and a wave takes as long: when the
+        // waves are fewer than one and a half for each of the chip's 1,024 SIMDs, two heads a wave: 46 -> 42 us.
+        // Asking for four pieces of a key row, or two groups of values, before the first is used: 112 us.)
+        int heads_a_wave = G <= 8 ? G : 4;
+        if (G > 8 && (long)slots * Hkv * ((G + 3) / 4) * num_rows < 1536) heads_a_wave = 2;
+        const int stretches = (G + heads_a_wave - 1) / heads_a_wave;
         RI_REQUIRE((long)Hkv * stretches <= 65535, "ri_attention_window: too many heads for the grid");
         part<<<dim3((slots + 3) / 4, Hkv * stretches, num_rows), 256, sizeof(float) * 4 * G * AD_KEYS, stream>>>(
             q, q_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, dk, dv, page, scale, window, slots, part_ml, part_o,

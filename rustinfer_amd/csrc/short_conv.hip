@@ -73,17 +73,26 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const ConvArgs a) {
         win[j] = j < hist ? (i0 == 0 ? old[j] : input(i)) : 0.f;
     }
     const int i1 = min(n, i0 + SC_CHUNK);
-    for (int i = i0; i < i1; ++i) {
-        const float cur = input(i);
-        float y = 0.f;
+    // eight inputs are asked for before the first is used: the loads of a chunk wait together, not in turn
+    for (int i8 = i0; i8 < i1; i8 += 8) {
+        float ahead[8];
 #pragma unroll
-        for (int j = 0; j < SC_MAX_TAPS - 1; ++j) if (j < hist) y = fmaf(w[j], win[j], y);
-        y = fmaf(w[hist], cur, y);
+        for (int u = 0; u < 8; ++u) ahead[u] = i8 + u < i1 ? input(i8 + u) : 0.f;
 #pragma unroll
-        for (int j = 0; j < SC_MAX_TAPS - 2; ++j) if (j + 1 < hist) win[j] = win[j + 1];
-        if (hist > 0) win[hist - 1] = cur;
-        if (a.silu) y = y / (1.f + expf(-y));
-        a.out[(size_t)(t_lo + i) * a.out_stride + oc] = y;
+        for (int u = 0; u < 8; ++u) {
+            const int i = i8 + u;
+            if (i >= i1) break;
+            const float cur = ahead[u];
+            float y = 0.f;
+#pragma unroll
+            for (int j = 0; j < SC_MAX_TAPS - 1; ++j) if (j < hist) y = fmaf(w[j], win[j], y);
+            y = fmaf(w[hist], cur, y);
+#pragma unroll
+            for (int j = 0; j < SC_MAX_TAPS - 2; ++j) if (j + 1 < hist) win[j] = win[j + 1];
+            if (hist > 0) win[hist - 1] = cur;
+            if (a.silu) y = y / (1.f + expf(-y));
+            a.out[(size_t)(t_lo + i) * a.out_stride + oc] = y;
+        }
     }
     if (i0 != 0) return;
     // the new state: the last taps - 1 inputs up to the row's last token, older ones from the old state
