@@ -235,7 +235,7 @@ def test_latent_attention_with_window_and_sink_alone(dtype, H, d, r, dv, R, dims
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("decoded", [False, True])
-@pytest.mark.parametrize("window", [16, 33, 136, 200])
+@pytest.mark.parametrize("window", [16, 33, 141, 200])
 def test_a_key_at_the_windows_edge_decides(dtype, decoded, window, portion_kernel):
     """Queries that match one key each: the key that lies window - 1 back is seen (the output is that
     key's value), the key that lies window back is not (the output is what the others and the sink leave).
