@@ -462,8 +462,10 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
     const int j = kb * AD_KEYS + lane;
     const bool mine = j >= j0 && j < visible;
     long long off = -1;
+    int own_pid = -1;                                  // the page of the lane's own key
     if (mine) {
         const int pid = table[(size_t)b * max_blocks + j / page];
+        own_pid = pid;
         if (pid >= 0) off = ((long long)pid * Hkv + g) * page + j % page;
     }
     const T* kr = off >= 0 ? kc + (size_t)off * dk : nullptr;
@@ -524,7 +526,9 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
 #pragma unroll
                 for (int c = 0; c < NC; ++c) v[u][c] = 0.f;
             if (vvec) {
-                const int pid = key + VL > j0 ? table[(size_t)b * max_blocks + key / page] : -1;
+                // the group's page from the lane of its first key that the row sees (the same page: VL keys
+                // do not cross one), not from the table again: a trip to memory less for every group
+                const int pid = key + VL > j0 ? __shfl(own_pid, max(jj, j0 - kb * AD_KEYS), 64) : -1;
                 if (pid >= 0) {
 #pragma unroll
                     for (int c = 0; c < NC; ++c) {
