@@ -580,3 +580,63 @@ def test_trace_replay_of_a_pilavik_model(tdirs, plain_logits, tmp_path):
         if n:
             results[st["step"]] = np.fromfile(os.path.join(str(tmp_path), f"{st['step']}.f32"), dtype="<f4").reshape(n, -1)
     check_rows(steps, results, logits, "bfloat16", "trace replay")
+
+
+# ---------------------------------------------------------------------------
+# configurations drawn at random
+# ---------------------------------------------------------------------------
+def draw_config(rng):
+    """A configuration whose every size, the order of its layers and its stretch are drawn: widths up to
+    1,024, up to 40 heads, keys of the latent up to 256 features, windows around page borders, up to 32
+    experts, convolutions of 1 to 8 taps, layers without feed-forward, a stretch anywhere or none."""
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+    layers = []
+    for _ in range(int(rng.integers(3, 8))):
+        if rng.random() < 0.55:
+            H = pick([1, 2, 4, 6, 8, 12, 16])
+            mixer = delta(H, pick([d for d in (1, 2, 3, 4, 6, 8, 16) if H % d == 0]), pick([16, 32, 48, 64, 96, 128]),
+                          pick([16, 32, 64, 128]), pick([1, 2, 3, 4, 5, 8]))
+        else:
+            r = pick([8, 16, 32, 64])
+            mixer = lat(pick([1, 2, 3, 4, 6, 8, 12, 16, 40]), pick([16, 32, 64, 128]), r, pick([16, 32, 64, 128]),
+                        pick([x for x in (32, 64, 128, 192) if x + r <= 256]), pick([0.1, 0.125, 0.2]),
+                        window=pick([None, 5, 16, 17, 48, 100, 128, 150, 256]), base=pick([100.0, 1e4, 3e5]),
+                        dims=r if rng.random() < 0.7 else r // 2)
+        k = rng.random()
+        if k < 0.15:
+            mlp = None
+        elif k < 0.55:
+            mlp = dense(pick([64, 200, 512, 1024, 2048]))
+        else:
+            E = pick([2, 4, 8, 16, 32])
+            mlp = moe(E, pick([t for t in (1, 2, 4, 8) if t <= E]), pick([16, 64, 128, 256]), scale=pick([1.0, 1.5, 2.5]),
+                      shared=pick([0, 0, 32, 128, 256]))
+        layers.append(layer(mixer, mlp))
+    cfg = dict(architecture="Pilavik", vocab=pick([100, 333, 777, 1000]), width=pick([64, 96, 192, 320, 512, 1024]),
+               norm=dict(eps=pick([1e-5, 1e-6])), layers=layers)
+    if rng.random() < 0.75:
+        a = int(rng.integers(0, len(layers)))
+        cfg["loop"] = dict(start=a, stop=int(rng.integers(a + 1, len(layers) + 1)), times=int(rng.integers(1, 4)))
+    return cfg
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15, 16])
+def test_configurations_drawn_at_random(seed, tmp_path):
+    """In 32-bit, where rounding hides nothing: last tokens alone, portions, and a mixed schedule on a pool
+    that is too small for all requests at once, against the plain implementation."""
+    from rustinfer_amd.engine import build_engine
+    from rustinfer_amd.weights import write_safetensors
+    cfg = draw_config(np.random.default_rng(seed))
+    w = draw_weights(cfg, seed)
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(cfg, f)
+    write_safetensors(str(tmp_path / "model.safetensors"), w)
+    reqs = random_requests(cfg["vocab"], (150, 3, 290, 40, 1, 77), seed)
+    logits = Rows({rid: P.forward(cfg, w, toks).numpy() for rid, toks in reqs.items()})
+    max_tokens = 2 * 320 + 64
+    eng = build_engine(str(tmp_path), dtype="float32", device=DEV, page_size=16, num_pages=max_tokens // 16, max_requests=4,
+                       max_model_len=max_tokens, max_batch_tokens=2048)
+    for label, steps in (("last tokens alone", cut_tail_single(reqs, tail=40)), ("portions", cut_portions(reqs, seed=seed)),
+                         ("mixed", cut_mixed(reqs, max_tokens, seed=seed, max_live=4, tail=6))):
+        check_rows(steps, run_steps(eng, steps), logits, "float32", f"{json.dumps(cfg)} {label}")
+        assert not eng.cache.live_requests()
