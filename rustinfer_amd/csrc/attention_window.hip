@@ -536,8 +536,13 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
                         if (d < dv) {
                             float f[VL];
                             ld_vec16(vc + (((size_t)pid * Hkv + g) * dv + d) * page + key % page, f);
+                            if (key >= j0 && key + VL <= visible) {      // (the same for the whole wave)
 #pragma unroll
-                            for (int u = 0; u < VL; ++u) v[u][c] = (key + u >= j0 && key + u < visible) ? f[u] : 0.f;
+                                for (int u = 0; u < VL; ++u) v[u][c] = f[u];
+                            } else {                                     // a group at the window's or the request's end
+#pragma unroll
+                                for (int u = 0; u < VL; ++u) v[u][c] = (key + u >= j0 && key + u < visible) ? f[u] : 0.f;
+                            }
                         }
                     }
                 }
