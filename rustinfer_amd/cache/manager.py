@@ -24,7 +24,7 @@ from typing import Dict, Hashable, List, Optional, Tuple
 import numpy as np
 import torch
 
-from ..parts.base import PagedKVNeed, StateNeed
+from ..parts.base import CompoundNeed, PagedKVNeed, StateNeed
 from .pages import CacheError, OutOfPages, PageAllocator
 
 
@@ -40,6 +40,17 @@ class KVCacheView:
     group: int               # index into StepContext.block_tables
     page_size: int
     write: bool
+
+
+@dataclass
+class CompoundView:
+    """What a layer with a ``CompoundNeed`` gets: its pages and its state."""
+    kv: KVCacheView
+    state: "StateView"
+
+    @property
+    def write(self) -> bool:
+        return self.kv.write
 
 
 @dataclass
@@ -74,16 +85,26 @@ class PageGroup:
         return self._np_tables[rid][:len(self.tables[rid])]
 
     def first_needed_page(self, next_pos: int) -> int:
-        """Pages below this index are no longer read once the next query is at ``next_pos``."""
+        """Pages below this index are no longer read by the window once the next query is at ``next_pos``."""
         if self.need.window is None:
             return 0
         return max(0, next_pos - self.need.window + 1) // self.page_size
 
+    @property
+    def kept_pages(self) -> int:
+        """The first pages of a request that are never given back: they hold positions every query may read."""
+        keep = getattr(self.need, "keep_first", 0) or 0
+        return pages_for(keep, self.page_size) if self.need.window is not None else 0
+
+    def droppable(self, next_pos: int) -> range:
+        """Indices of the table entries no query at ``next_pos`` or later reads."""
+        return range(self.kept_pages, max(self.kept_pages, self.first_needed_page(next_pos)))
+
     def new_pages_for(self, rid, kv_len: int, n: int) -> Tuple[int, int]:
         """(pages to take, pages to give back first) for appending ``n`` tokens at ``kv_len``."""
         table = self.tables[rid]
-        drop_below = self.first_needed_page(kv_len)
-        give_back = sum(1 for p in table[:drop_below] if p >= 0)
+        drop = self.droppable(kv_len)
+        give_back = sum(1 for p in table[drop.start:drop.stop] if p >= 0)
         take = max(0, pages_for(kv_len + n, self.page_size) - len(table))
         return take, give_back
 
@@ -109,25 +130,30 @@ class CacheManager:
         by_need: Dict[PagedKVNeed, List[int]] = {}
         self.state_tensors: Dict[object, torch.Tensor] = {}      # cache id (or (cache id, name) of a further tensor) -> [slots, ...]
         self._state_extra: Dict[int, List[str]] = {}
+        self._kv_where: Dict[int, Tuple[int, int]] = {}       # cache id -> (group, layer slot) of a compound need's pages
         for cid in sorted(needs):
             need = needs[cid]
-            if isinstance(need, PagedKVNeed):
-                by_need.setdefault(need, []).append(cid)
-            elif isinstance(need, StateNeed):
-                self._where[cid] = ("state", cid, 0)
+            kv_need = need.kv if isinstance(need, CompoundNeed) else need if isinstance(need, PagedKVNeed) else None
+            state_need = need.state if isinstance(need, CompoundNeed) else need if isinstance(need, StateNeed) else None
+            if kv_need is None and state_need is None:
+                raise TypeError(f"cache {cid}: unknown need {need!r}")
+            if kv_need is not None:
+                by_need.setdefault(kv_need, []).append(cid)
+            if state_need is not None:
+                self._where[cid] = ("both" if kv_need is not None else "state", cid, 0)
                 if device is not None:
                     # one slot more than requests: the scratch slot of rows that belong to no request
-                    for name, shape, state_dtype in need.all_tensors():
+                    for name, shape, state_dtype in state_need.all_tensors():
                         self.state_tensors[(cid, name) if name else cid] = torch.zeros((max_requests + 1,) + shape,
                                                                                     device=device, dtype=state_dtype)
-                self._state_extra[cid] = [name for name, _, _ in need.extra]
-            else:
-                raise TypeError(f"cache {cid}: unknown need {need!r}")
+                self._state_extra[cid] = [name for name, _, _ in state_need.extra]
         for gi, (need, cids) in enumerate(by_need.items()):
             self.groups.append(PageGroup(gi, need, cids, page_size, num_pages, max_model_len,
                                          device, dtype))
             for slot, cid in enumerate(cids):
-                self._where[cid] = ("kv", gi, slot)
+                self._kv_where[cid] = (gi, slot)
+                if cid not in self._where:
+                    self._where[cid] = ("kv", gi, slot)
         self.slots = PageAllocator(max_requests, what="slots")
         # Rows of a step that belong to no request (padding of a captured batch size, the rows a
         # graph is warmed up and captured on) point here: a mixer that updates state in place may
@@ -164,11 +190,16 @@ class CacheManager:
 
     def view(self, cache_id: int, write: bool = True):
         kind, where, slot = self._where[cache_id]
-        if kind == "kv":
-            g = self.groups[where]
-            return KVCacheView(g.k_pool[slot], g.v_pool[slot], g.index, g.page_size, write)
-        names = self._state_extra.get(where) or []
-        return StateView(self.state_tensors[where], write, {n: self.state_tensors[(where, n)] for n in names} if names else None)
+        kv = None
+        if kind in ("kv", "both"):
+            gi, slot = self._kv_where[cache_id]
+            g = self.groups[gi]
+            kv = KVCacheView(g.k_pool[slot], g.v_pool[slot], g.index, g.page_size, write)
+            if kind == "kv":
+                return kv
+        names = self._state_extra.get(cache_id) or []
+        state = StateView(self.state_tensors[cache_id], write, {n: self.state_tensors[(cache_id, n)] for n in names} if names else None)
+        return CompoundView(kv, state) if kv is not None else state
 
     # -- life of a request -----------------------------------------------------
     def add_request(self, rid) -> int:
@@ -219,13 +250,14 @@ class CacheManager:
                 raise OutOfPages(take, g.allocator.available + give)
         for g in self.groups:
             table = g.tables[rid]
-            drop_below = g.first_needed_page(start)
-            old = [p for p in table[:drop_below] if p >= 0]
+            drop = g.droppable(start)
+            lo, hi = min(drop.start, len(table)), min(drop.stop, len(table))
+            old = [p for p in table[lo:hi] if p >= 0]
             if old:
                 g.allocator.free(old)
-                for i in range(min(drop_below, len(table))):
+                for i in range(lo, hi):
                     table[i] = -1
-                g._np_tables[rid][:min(drop_below, len(table))] = -1
+                g._np_tables[rid][lo:hi] = -1
             take = max(0, pages_for(start + n, g.page_size) - len(table))
             if take:
                 new = g.allocator.alloc(take)
@@ -245,7 +277,8 @@ class CacheManager:
             raise CacheError(f"request {rid!r}: cannot truncate {self._kv_len[rid]} tokens to {length}")
         for g in self.groups:
             keep = pages_for(length, g.page_size)
-            if any(p < 0 for p in g.tables[rid][g.first_needed_page(length):keep]):
+            if any(p < 0 for p in g.tables[rid][g.first_needed_page(length):keep]) \
+                    or any(p < 0 for p in g.tables[rid][:min(g.kept_pages, keep)]):
                 raise CacheError(f"request {rid!r}: a window has given back pages that a query at "
                                  f"position {length} reads; it cannot be cut back that far")
         for g in self.groups:

@@ -917,3 +917,285 @@ class PilavikConfig(ModelConfig):
         if self.eos_token_ids:
             d["eos_token_id"] = list(self.eos_token_ids)
         return d
+
+
+# ---------------------------------------------------------------------------
+# Debuzen: pre-norm layers with a norm in groups and a token shift in front of the mixer; mixers that are
+# two sub-mixers side by side (attention and a recurrence) or gated linear attention; a stretch of
+# layers that runs several times behind a product over the stream and the embedded rows
+# ---------------------------------------------------------------------------
+DEFAULT_LOW_RANK = 16     # rows of the first of two matrices that make a decay's or a gate's input, where no checkpoint says
+
+
+def _mask_of(m: Dict[str, Any], where: str):
+    """(size, keep_first) of a mixer's 'mask' object."""
+    mask = _obj(m, "mask", where)
+    size = _require(mask, "size", int, where + ".mask")
+    keep = _typed(mask.get("keep_first", 0), "keep_first", int, where + ".mask")
+    if size <= 0 or keep < 0:
+        raise ConfigError(f"{where}.mask: size must be > 0 and keep_first >= 0")
+    return size, keep
+
+
+@dataclass(frozen=True)
+class MaskedAttentionSpec:
+    """The attention half of a mixer of two: grouped heads (keys of ``dim``, values of ``vdim``), a rotation
+    over the first ``rot_dims`` features, a sliding window of ``window`` positions behind which the first
+    ``keep_first`` positions of a sequence stay in sight."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int
+    keep_first: int
+    rot_base: float
+    rot_dims: int
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "MaskedAttentionSpec":
+        base, dims, scaling = _rot_of(m, where)
+        if scaling is not None:
+            raise ConfigError(f"{where}.rot: this design's rotation is not stretched")
+        size, keep = _mask_of(m, where)
+        s = MaskedAttentionSpec(heads=_require(m, "heads", int, where), kv_heads=_require(m, "kv_heads", int, where),
+                                dim=_require(m, "dim", int, where), vdim=_require(m, "vdim", int, where),
+                                scale=_require(m, "scale", float, where), window=size, keep_first=keep,
+                                rot_base=base, rot_dims=dims)
+        if min(s.heads, s.kv_heads, s.dim, s.vdim) <= 0 or s.heads % s.kv_heads:
+            raise ConfigError(f"{where}: heads, kv_heads, dim and vdim must be > 0 and heads a multiple of kv_heads")
+        if s.rot_dims > s.dim or max(s.dim, s.vdim) > MAX_HEAD_DIM:
+            raise ConfigError(f"{where}: rot.dims {s.rot_dims} exceeds dim {s.dim}, or a head exceeds {MAX_HEAD_DIM} features")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        mask = {"size": self.window}
+        if self.keep_first:
+            mask["keep_first"] = self.keep_first
+        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale,
+                "mask": mask, "rot": _rot_dict(self.rot_base, self.rot_dims)}
+
+
+@dataclass(frozen=True)
+class ChannelDeltaSpec:
+    """The gated delta rule with a decay for every key channel; the decay's and the gate's inputs come through
+    two matrices each, whose inner sizes (``decay_rank``, ``gate_rank``) the checkpoint's shapes give."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    decay_rank: int = DEFAULT_LOW_RANK
+    gate_rank: int = DEFAULT_LOW_RANK
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "ChannelDeltaSpec":
+        s = ChannelDeltaSpec(heads=_require(m, "heads", int, where), kv_heads=_require(m, "kv_heads", int, where),
+                             dim=_require(m, "dim", int, where), vdim=_require(m, "vdim", int, where),
+                             conv=_require(m, "conv", int, where),
+                             decay_rank=_typed(m.get("decay_rank", DEFAULT_LOW_RANK), "decay_rank", int, where),
+                             gate_rank=_typed(m.get("gate_rank", DEFAULT_LOW_RANK), "gate_rank", int, where))
+        if min(s.heads, s.kv_heads, s.dim, s.vdim, s.conv, s.decay_rank, s.gate_rank) <= 0 or s.heads % s.kv_heads:
+            raise ConfigError(f"{where}: every size must be > 0 and heads a multiple of kv_heads")
+        if s.dim > MAX_HEAD_DIM or s.conv > 8:
+            raise ConfigError(f"{where}: dim {s.dim} exceeds {MAX_HEAD_DIM} or conv {s.conv} exceeds 8 taps")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "conv": self.conv}
+
+
+@dataclass(frozen=True)
+class StateSpaceSpec:
+    """A state-space mixer in its recurrent form: ``heads`` heads of ``vdim`` over a state of ``state`` rows,
+    inputs shared by ``groups`` groups of heads, a convolution of ``conv`` taps, an output norm in
+    ``norm_groups`` parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int
+
+    @staticmethod
+    def from_dict(m: Dict[str, Any], where: str) -> "StateSpaceSpec":
+        s = StateSpaceSpec(heads=_require(m, "heads", int, where), vdim=_require(m, "vdim", int, where),
+                           state=_require(m, "state", int, where), groups=_require(m, "groups", int, where),
+                           conv=_require(m, "conv", int, where), norm_groups=_require(m, "norm_groups", int, where))
+        if min(s.heads, s.vdim, s.state, s.groups, s.conv, s.norm_groups) <= 0 or s.heads % s.groups \
+                or (s.heads * s.vdim) % s.norm_groups:
+            raise ConfigError(f"{where}: every size must be > 0, heads a multiple of groups, heads * vdim of norm_groups")
+        if s.state > MAX_HEAD_DIM or s.conv > 8:
+            raise ConfigError(f"{where}: state {s.state} exceeds {MAX_HEAD_DIM} or conv {s.conv} exceeds 8 taps")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"heads": self.heads, "vdim": self.vdim, "state": self.state, "groups": self.groups, "conv": self.conv,
+                "norm_groups": self.norm_groups}
+
+
+@dataclass(frozen=True)
+class TwoMixerSpec:
+    """Mixers ``parallel`` (attention with sigmoid weights and kept first positions beside the channel-gated
+    delta rule) and ``parallel_2`` (softmax attention with a sink beside a state-space mixer): both halves read
+    the same rows, and the result is ``left_scale * left + right_scale * right``."""
+    kind: str
+    left: MaskedAttentionSpec
+    right: Any
+    left_scale: float
+    right_scale: float
+
+    @staticmethod
+    def from_dict(kind: str, m: Dict[str, Any], where: str) -> "TwoMixerSpec":
+        right_cls = ChannelDeltaSpec if kind == "parallel" else StateSpaceSpec
+        s = TwoMixerSpec(kind, MaskedAttentionSpec.from_dict(_obj(m, "left", where), where + ".left"),
+                         right_cls.from_dict(_obj(m, "right", where), where + ".right"),
+                         _require(m, "left_scale", float, where), _require(m, "right_scale", float, where))
+        if kind == "parallel_2" and s.left.keep_first:
+            raise ConfigError(f"{where}.left.mask: the softmax half keeps no first positions")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"left": self.left.to_dict(), "right": self.right.to_dict(), "left_scale": self.left_scale,
+                "right_scale": self.right_scale}
+
+
+@dataclass(frozen=True)
+class GatedLinearSpec:
+    """Mixer ``gla``: gated linear attention, a decay ``sigmoid(.)^(1 / tau)`` for every key channel whose input
+    comes through two matrices (inner size ``decay_rank``, from the checkpoint's shapes)."""
+    heads: int
+    dim: int
+    vdim: int
+    tau: float
+    decay_rank: int = DEFAULT_LOW_RANK
+    kind: str = "gla"
+
+    @staticmethod
+    def from_dict(kind: str, m: Dict[str, Any], where: str) -> "GatedLinearSpec":
+        s = GatedLinearSpec(heads=_require(m, "heads", int, where), dim=_require(m, "dim", int, where),
+                            vdim=_require(m, "vdim", int, where), tau=_require(m, "tau", float, where),
+                            decay_rank=_typed(m.get("decay_rank", DEFAULT_LOW_RANK), "decay_rank", int, where))
+        if min(s.heads, s.dim, s.vdim, s.decay_rank) <= 0 or not s.tau > 0 or s.dim > MAX_HEAD_DIM:
+            raise ConfigError(f"{where}: heads, dim, vdim and tau must be > 0 and dim at most {MAX_HEAD_DIM}")
+        return s
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "tau": self.tau}
+
+
+DEBUZEN_MIXERS = {"parallel": TwoMixerSpec, "parallel_2": TwoMixerSpec, "gla": GatedLinearSpec}
+
+
+@dataclass(frozen=True)
+class DebuzenLayer:
+    mixer: Any                    # TwoMixerSpec or GatedLinearSpec
+    ff: Optional[int] = None      # width of the gated feed-forward; None: the layer has none
+
+    @property
+    def type(self) -> str:
+        return self.mixer.kind
+
+
+@dataclass(frozen=True)
+class DebuzenConfig(ModelConfig):
+    """``{"architecture": "Debuzen", "vocab", "width", "norm": {"eps", "groups"}, "logit_softcap", "layers":
+    [{"type", "mixer": {...}, "mlp": {"kind": "dense", "ff"} | null}], "loop": {"start", "stop", "times"} |
+    absent}``.  Every norm works in ``norm.groups`` equal parts of a row.  Layers ``start .. stop - 1`` run
+    ``times`` times in a row with the same weights, each pass on a cache and state of its own, behind a
+    product of the stream and the embedded rows; the head has a matrix of its own."""
+
+    vocab_size: int = 0
+    hidden_size: int = 0
+    norm_eps: float = 1e-6
+    norm_groups: int = 1
+    logit_softcap: float = 0.0
+    layers: tuple = ()
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    has_loop: bool = False
+    eos_token_ids: tuple = ()
+    architecture: str = "Debuzen"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any], where: str = "config.json") -> "DebuzenConfig":
+        layers_in = d.get("layers")
+        if not isinstance(layers_in, list) or not layers_in:
+            raise ConfigError(f"{where}: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(layers_in):
+            w = f"{where}.layers[{i}]"
+            if not isinstance(entry, dict):
+                raise ConfigError(f"{w}: must be an object")
+            kind = _require(entry, "type", str, w)
+            if kind not in DEBUZEN_MIXERS:
+                raise ConfigError(f"{w}: unknown mixer type {kind!r} (known: {', '.join(sorted(DEBUZEN_MIXERS))})")
+            mixer = DEBUZEN_MIXERS[kind].from_dict(kind, _obj(entry, "mixer", w), w + ".mixer")
+            mlp = entry.get("mlp")
+            ff = None
+            if mlp is not None:
+                if not isinstance(mlp, dict):
+                    raise ConfigError(f"{w}: 'mlp' must be null or an object")
+                if mlp.get("kind", "dense") != "dense":
+                    raise ConfigError(f"{w}.mlp: unknown feed-forward kind {mlp.get('kind')!r} (known: dense)")
+                ff = _require(mlp, "ff", int, w + ".mlp")
+                if ff <= 0:
+                    raise ConfigError(f"{w}.mlp: ff must be > 0")
+            layers.append(DebuzenLayer(mixer, ff))
+        loop = d.get("loop")
+        start = stop = 0
+        times = 1
+        if loop is not None:
+            if not isinstance(loop, dict):
+                raise ConfigError(f"{where}: 'loop' must be an object or null")
+            w = where + ".loop"
+            start, stop, times = _require(loop, "start", int, w), _require(loop, "stop", int, w), _require(loop, "times", int, w)
+            if not (0 <= start < stop <= len(layers)) or times < 1:
+                raise ConfigError(f"{w}: need 0 <= start < stop <= {len(layers)} layers and times >= 1")
+        norm = _obj(d, "norm", where)
+        eos = d.get("eos_token_id")
+        eos_ids = () if eos is None else tuple(_typed(e, "eos_token_id", int, where) for e in (eos if isinstance(eos, list) else [eos]))
+        cfg = cls(vocab_size=_require(d, "vocab", int, where), hidden_size=_require(d, "width", int, where),
+                  norm_eps=_require(norm, "eps", float, where + ".norm"),
+                  norm_groups=_typed(norm.get("groups", 1), "groups", int, where + ".norm"),
+                  logit_softcap=_typed(d.get("logit_softcap", 0.0) or 0.0, "logit_softcap", float, where),
+                  layers=tuple(layers), loop_start=start, loop_stop=stop, loop_times=times, has_loop=loop is not None,
+                  eos_token_ids=eos_ids)
+        if cfg.vocab_size <= 0 or cfg.hidden_size <= 0 or not cfg.norm_eps > 0 or cfg.logit_softcap < 0:
+            raise ConfigError(f"{where}: vocab and width must be > 0, norm.eps > 0, logit_softcap >= 0")
+        if cfg.norm_groups <= 0 or cfg.hidden_size % cfg.norm_groups:
+            raise ConfigError(f"{where}.norm: width {cfg.hidden_size} does not split into {cfg.norm_groups} equal parts")
+        return cfg
+
+    def complete_from_checkpoint(self, shapes: Dict[str, Any]) -> "DebuzenConfig":
+        """The sizes that only a tensor's shape gives (``shapes``: checkpoint name -> shape): the inner sizes
+        of the pairs of matrices that make decays and gates (rows of ``a1`` and ``g1``)."""
+        from dataclasses import replace
+
+        def rows(name, default):
+            shape = shapes.get(name)
+            return int(shape[0]) if shape is not None and len(shape) == 2 else default
+
+        layers = []
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            if isinstance(m, GatedLinearSpec):
+                m = replace(m, decay_rank=rows(f"l{i}.mix.a1", m.decay_rank))
+            elif isinstance(m.right, ChannelDeltaSpec):
+                m = replace(m, right=replace(m.right, decay_rank=rows(f"l{i}.mix.right.a1", m.right.decay_rank),
+                                             gate_rank=rows(f"l{i}.mix.right.g1", m.right.gate_rank)))
+            layers.append(DebuzenLayer(m, layer.ff))
+        return replace(self, layers=tuple(layers))
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {
+            "architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+            "norm": {"eps": self.norm_eps, "groups": self.norm_groups}, "logit_softcap": self.logit_softcap,
+            "layers": [{"type": l.type, "mixer": l.mixer.to_dict(),
+                        "mlp": None if l.ff is None else {"kind": "dense", "ff": l.ff}} for l in self.layers]}
+        if self.has_loop:
+            d["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids)
+        return d

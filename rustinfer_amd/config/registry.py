@@ -103,3 +103,4 @@ def _ensure_builtin() -> None:
     from ..models import tedelix  # noqa: F401  (registers Tedelix)
     from ..models import belorax  # noqa: F401  (registers Belorax)
     from ..models import pilavik  # noqa: F401  (registers Pilavik)
+    from ..models import debuzen  # noqa: F401  (registers Debuzen)

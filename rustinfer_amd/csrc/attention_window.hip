@@ -32,6 +32,7 @@
 namespace {
 
 constexpr int AW_ROWS = 32;
+constexpr int AW_NORM_HEADS = 1024;   // query and key heads whose unit factors rotate_kv_write holds
 
 template <typename T>
 __global__ __launch_bounds__(256) void rotate_kv_write_kernel(
@@ -39,30 +40,53 @@ __global__ __launch_bounds__(256) void rotate_kv_write_kernel(
         int H, int Hkv, int dk, int dv, int rot, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
         const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved,
         const int* __restrict__ positions, const int* __restrict__ row_of_token,
-        T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ table, int max_blocks, int page, int write_kv) {
+        T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ table, int max_blocks, int page, int write_kv,
+        float unit_eps) {
+    __shared__ float inv[AW_NORM_HEADS];     // unit_eps > 0: 1 / root mean square of every query head, then of every key head
     const int t = blockIdx.x;
     const int b = row_of_token[t];
     if (b < 0) return;                       // padding token
     const int pos = positions[t];
     const int half = rot >> 1;
     const bool rotate = cos_t != nullptr;
+    const bool unit = unit_eps > 0.f;
     const float* cs = rotate ? cos_t + (size_t)pos * half : nullptr;
     const float* sn = rotate ? sin_t + (size_t)pos * half : nullptr;
     T* qrow = q + (size_t)t * q_stride;
+    const T* krow = k + (size_t)t * k_stride;
+    if (unit) {
+        // a rotation leaves a head's sum of squares as it is: the factors are made from the rows as projected
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int nk = write_kv ? Hkv : 0;
+        for (int h = wave; h < H + nk; h += 4) {
+            const T* row = h < H ? qrow + h * dk : krow + (h - H) * dk;
+            float ss = 0.f;
+            for (int d = lane; d < dk; d += 64) { const float x = ld_f32(row + d); ss = fmaf(x, x, ss); }
+            ss = wave_sum(ss);
+            if (lane == 0) inv[h] = 1.f / sqrtf(ss / (float)dk + unit_eps);
+        }
+        __syncthreads();
+    }
     const int q_pairs = rotate ? H * half : 0;
     for (int idx = threadIdx.x; idx < q_pairs; idx += 256) {
         const int h = idx / half, i = idx - h * half;
         T* qh = qrow + h * dk;
         const float a = ld_f32(qh + i), bb = ld_f32(qh + i + half);
-        const float c = cs[i], s = sn[i];
-        st_f32(qh + i, a * c - bb * s);
-        st_f32(qh + i + half, bb * c + a * s);
+        const float c = cs[i], s = sn[i], f = unit ? inv[h] : 1.f;
+        st_f32(qh + i, (a * c - bb * s) * f);
+        st_f32(qh + i + half, (bb * c + a * s) * f);
+    }
+    if (unit) {
+        const int first = rotate ? rot : 0, rest = dk - first;        // the features that are not turned
+        for (int idx = threadIdx.x; idx < H * rest; idx += 256) {
+            const int h = idx / rest, d = first + idx - h * rest;
+            st_f32(qrow + h * dk + d, ld_f32(qrow + h * dk + d) * inv[h]);
+        }
     }
     if (!write_kv) return;
     const int blk = table[(size_t)b * max_blocks + pos / page];
     if (blk < 0) return;
     const int slot = pos % page;
-    const T* krow = k + (size_t)t * k_stride;
     for (int idx = threadIdx.x; idx < Hkv * dk; idx += 256) {
         const int g = idx / dk, dd = idx - g * dk;
         const T* kh = krow + g * dk;
@@ -70,6 +94,7 @@ __global__ __launch_bounds__(256) void rotate_kv_write_kernel(
         if (rotate && dd < half) val = ld_f32(kh + dd) * cs[dd] - ld_f32(kh + dd + half) * sn[dd];
         else if (rotate && dd < rot) val = ld_f32(kh + dd) * cs[dd - half] + ld_f32(kh + dd - half) * sn[dd - half];
         else val = ld_f32(kh + dd);
+        if (unit) val *= inv[H + g];
         st_f32(kc + (((size_t)blk * Hkv + g) * page + slot) * dk + dd, val);
     }
     const T* vrow = v + (size_t)t * v_stride;
@@ -101,6 +126,16 @@ __device__ __forceinline__ float aw_block_scores(float dot, bool mine, float sca
     m_b = wave_max(sc);
     float pj = 0.f;
     if (m_b > -INFINITY) pj = mine ? expf(sc - m_b) : 0.f;
+    l_b = wave_sum(pj);
+    return pj;
+}
+
+// The same for weights that are sigmoids of the scores plus a number a head, with no normalisation over
+// the keys: the block's "maximum" is 0 where the row sees a key of it, so that merging adds the blocks' sums
+// as they are (exp(0 - 0) = 1), and the result is the sum itself (aw_final_factor gives 1).
+__device__ __forceinline__ float aw_block_sigmoids(float dot, bool mine, float scale, float bias, float& m_b, float& l_b) {
+    const float pj = mine ? 1.f / (1.f + expf(-(dot * scale + bias))) : 0.f;
+    m_b = __any(mine) ? 0.f : -INFINITY;
     l_b = wave_sum(pj);
     return pj;
 }
@@ -146,7 +181,8 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
         const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int num_rows, int H, int Hkv, int dk, int dv, int page, float scale, int window, int TQ, int NK,
-        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved, const float* __restrict__ sink) {
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved, const float* __restrict__ sink,
+        int keep, const float* __restrict__ sig_bias) {
     extern __shared__ __align__(16) float lds[];
     const int dkp = (dk + 3) & ~3, ks_stride = dkp + 4, vs_stride = dv + 1;
     float* Qs = lds;                                   // [AW_ROWS][dkp]
@@ -194,13 +230,15 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
         row_lo[i] = window > 0 ? max(0, p + 1 - window) : 0;
     }
 
-    for (int kb = first_key / NK; kb * NK < last_visible; ++kb) {
+    // keep > 0: the first `keep` positions stay in sight behind the window: their blocks of keys first
+    for (int kb = keep > 0 ? 0 : first_key / NK; kb * NK < last_visible; ++kb) {
+        if (kb * NK >= keep && kb < first_key / NK) kb = first_key / NK;      // from the kept positions on to the window
         const int j_base = kb * NK;
         __syncthreads();                               // the last block of keys has been used (first pass: Qs is written)
         if (tid < NK) {
             const int j = j_base + tid;
             int off = -1;
-            if (j < last_visible && j >= first_key) {
+            if (j < last_visible && (j >= first_key || j < keep)) {
                 const int pid = table[(size_t)b * max_blocks + j / page];
                 if (pid >= 0) off = (pid * Hkv + g) * page + j % page;      // -1: a page the window has given back
             }
@@ -284,8 +322,9 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 #pragma unroll
             for (int rb = 0; rb < 4; ++rb) {
                 const int i = 4 * bi + rb;
-                const bool mine = lane < NK && j >= row_lo[i] && j < row_hi[i];
-                const float pj = aw_block_scores(s[rb], mine, scale, m_b[i], l_b[i]);
+                const bool mine = lane < NK && (j >= row_lo[i] || j < keep) && j < row_hi[i];
+                const float pj = sig_bias ? aw_block_sigmoids(s[rb], mine, scale, sig_bias[g * G + (wave + 4 * i) % G], m_b[i], l_b[i])
+                                          : aw_block_scores(s[rb], mine, scale, m_b[i], l_b[i]);
                 if (lane < NK) Ps[(wave + 4 * i) * NK + lane] = pj;
             }
         }
@@ -326,11 +365,11 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
             const int r = wave + 4 * i;
             if (r >= R) continue;
             T* o = out + (size_t)(t0 + r / G) * out_stride + (g * G + r % G) * dv;
-            const float fin = sink ? aw_final_factor(m[i], l[i], sink, g * G + r % G) : 0.f;
+            const float fin = sig_bias ? 1.f : sink ? aw_final_factor(m[i], l[i], sink, g * G + r % G) : 0.f;
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 const int d = lane + 64 * c;
-                if (d < dv) st_f32(o + d, sink ? acc[i][c] * fin : (l[i] > 0.f ? acc[i][c] / l[i] : 0.f));
+                if (d < dv) st_f32(o + d, (sink || sig_bias) ? acc[i][c] * fin : (l[i] > 0.f ? acc[i][c] / l[i] : 0.f));
             }
         }
         return;
@@ -345,7 +384,7 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int d = lane + 64 * c;
-            if (d < dv) Os[r * dv + d] = sink ? acc[i][c] * aw_final_factor(m[i], l[i], sink, g * G + r % G) : (l[i] > 0.f ? acc[i][c] / l[i] : 0.f);
+            if (d < dv) Os[r * dv + d] = sig_bias ? acc[i][c] : sink ? acc[i][c] * aw_final_factor(m[i], l[i], sink, g * G + r % G) : (l[i] > 0.f ? acc[i][c] / l[i] : 0.f);
         }
     }
     __syncthreads();
@@ -363,6 +402,13 @@ __global__ __launch_bounds__(256) void attn_window_kernel(
     }
 }
 
+// Single tokens with kept first positions: how many of the blocks of NK keys that hold kept positions lie
+// wholly before the window's first block and hold a key the row sees (the others are the window's, or empty).
+__device__ __forceinline__ int aw_keep_used(int keep, int NK, int first_key, int visible) {
+    const int seen = min(keep, visible);
+    return min((seen + NK - 1) / NK, first_key / NK);
+}
+
 // Steps of single tokens: merge the partial results of a row's blocks of keys in ascending order
 // (the order and the arithmetic of the loop in attn_window_kernel), divide, turn back, write.
 // One wave a (token, head).
@@ -371,7 +417,8 @@ __global__ __launch_bounds__(64) void attn_window_combine_kernel(
         const float* __restrict__ part_ml, const float* __restrict__ part_o, T* __restrict__ out, int out_stride,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int H, int dv, int window, int NK, int slots,
-        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved, const float* __restrict__ sink) {
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved, const float* __restrict__ sink,
+        int keep, int sigmoid_weights) {
     __shared__ float Os[256];
     const int b = blockIdx.y, h = blockIdx.x, lane = threadIdx.x;
     const int t = cu_q[b];
@@ -379,7 +426,9 @@ __global__ __launch_bounds__(64) void attn_window_combine_kernel(
     const int p = q_start[b];
     const int visible = min(kv_lens[b], p + 1);
     const int first_key = window > 0 ? max(0, p + 1 - window) : 0;
-    const int n = (visible + NK - 1) / NK - first_key / NK;
+    // the first slots belong to the blocks of the kept positions (those that lie before the window's first block)
+    const int keep_slots = (keep + NK - 1) / NK, keep_used = aw_keep_used(keep, NK, first_key, visible);
+    const int n = keep_slots + (visible + NK - 1) / NK - first_key / NK;
     float m = -INFINITY, l = 0.f, acc[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) acc[c] = 0.f;
@@ -391,8 +440,8 @@ __global__ __launch_bounds__(64) void attn_window_combine_kernel(
         float acc_b[AHEAD][NC], m_b[AHEAD], l_b[AHEAD];
 #pragma unroll
         for (int i = 0; i < AHEAD; ++i) {
-            const bool on = s0 + i < count;
-            const size_t at = ((size_t)t * H + h) * slots + (on ? s0 + i : s0);
+            const bool on = s0 + i < count && (s0 + i >= keep_slots || s0 + i < keep_used);
+            const size_t at = ((size_t)t * H + h) * slots + (on ? s0 + i : 0);
             m_b[i] = on ? part_ml[at * 2] : -INFINITY;
             l_b[i] = on ? part_ml[at * 2 + 1] : 0.f;
 #pragma unroll
@@ -403,14 +452,14 @@ __global__ __launch_bounds__(64) void attn_window_combine_kernel(
         }
 #pragma unroll
         for (int i = 0; i < AHEAD; ++i)
-            if (s0 + i < count) aw_merge<NC>(m, l, acc, m_b[i], l_b[i], acc_b[i]);
+            if (s0 + i < count) aw_merge<NC>(m, l, acc, m_b[i], l_b[i], acc_b[i]);        // (a slot that is off has m_b = -inf)
     }
     T* o = out + (size_t)t * out_stride + h * dv;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
         const int d = lane + 64 * c;
         if (d < dv) {
-            const float y = sink ? acc[c] * aw_final_factor(m, l, sink, h) : (l > 0.f ? acc[c] / l : 0.f);
+            const float y = sigmoid_weights ? acc[c] : sink ? acc[c] * aw_final_factor(m, l, sink, h) : (l > 0.f ? acc[c] / l : 0.f);
             if (vcos == nullptr) st_f32(o + d, y);
             else Os[d] = y;
         }
@@ -440,7 +489,7 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
         const T* __restrict__ q, int q_stride, const T* __restrict__ kc, const T* __restrict__ vc,
         const int* __restrict__ table, int max_blocks, const int* __restrict__ cu_q, const int* __restrict__ q_start,
         const int* __restrict__ kv_lens, int H, int Hkv, int dk, int dv, int page, float scale, int window, int slots,
-        float* __restrict__ part_ml, float* __restrict__ part_o, int heads_a_wave) {
+        float* __restrict__ part_ml, float* __restrict__ part_o, int heads_a_wave, int keep, const float* __restrict__ sig_bias) {
     extern __shared__ __align__(16) float lds[];       // [4 waves][G][64] weights
     // many query heads a key/value head (one shared latent, say): the heads are dealt to several
     // blocks in stretches of heads_a_wave, each reading the block of keys for its own heads
@@ -454,13 +503,15 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
     const int visible = min(kv_lens[b], p + 1);
     const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
     const int slot = (int)blockIdx.x * 4 + wave;
-    const int kb = j0 / AD_KEYS + slot;
+    const int keep_slots = (keep + AD_KEYS - 1) / AD_KEYS;
+    if (slot < keep_slots && slot >= aw_keep_used(keep, AD_KEYS, j0, visible)) return;
+    const int kb = slot < keep_slots ? slot : j0 / AD_KEYS + slot - keep_slots;
     if (slot >= slots || kb * AD_KEYS >= visible) return;
     float* Ps = lds + (size_t)wave * G * AD_KEYS;
     constexpr int VL = 16 / sizeof(T);
 
     const int j = kb * AD_KEYS + lane;
-    const bool mine = j >= j0 && j < visible;
+    const bool mine = (j >= j0 || j < keep) && j < visible;
     long long off = -1;
     int own_pid = -1;                                  // the page of the lane's own key
     if (mine) {
@@ -501,7 +552,8 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
         for (int rb = 0; rb < 4; ++rb) {
             if (h0 + rb >= h_hi) break;
             float m_b, l_b;
-            Ps[(h0 + rb) * AD_KEYS + lane] = aw_block_scores(s[rb], mine, scale, m_b, l_b);
+            Ps[(h0 + rb) * AD_KEYS + lane] = sig_bias ? aw_block_sigmoids(s[rb], mine, scale, sig_bias[g * G + h0 + rb], m_b, l_b)
+                                                      : aw_block_scores(s[rb], mine, scale, m_b, l_b);
             if (lane == 0) {
                 float* dst = part_ml + (at0 + (size_t)(h0 + rb) * slots) * 2;
                 dst[0] = m_b;
@@ -528,7 +580,7 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
             if (vvec) {
                 // the group's page from the lane of its first key that the row sees (the same page: VL keys
                 // do not cross one), not from the table again: a trip to memory less for every group
-                const int pid = key + VL > j0 ? __shfl(own_pid, max(jj, j0 - kb * AD_KEYS), 64) : -1;
+                const int pid = key < keep ? __shfl(own_pid, jj, 64) : key + VL > j0 ? __shfl(own_pid, max(jj, j0 - kb * AD_KEYS), 64) : -1;
                 if (pid >= 0) {
 #pragma unroll
                     for (int c = 0; c < NC; ++c) {
@@ -536,12 +588,12 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
                         if (d < dv) {
                             float f[VL];
                             ld_vec16(vc + (((size_t)pid * Hkv + g) * dv + d) * page + key % page, f);
-                            if (key >= j0 && key + VL <= visible) {      // (the same for the whole wave)
+                            if ((key >= j0 || key + VL <= keep) && key + VL <= visible) {      // (the same for the whole wave)
 #pragma unroll
                                 for (int u = 0; u < VL; ++u) v[u][c] = f[u];
-                            } else {                                     // a group at the window's or the request's end
+                            } else {                                     // a group at the window's, the kept positions' or the request's end
 #pragma unroll
-                                for (int u = 0; u < VL; ++u) v[u][c] = (key + u >= j0 && key + u < visible) ? f[u] : 0.f;
+                                for (int u = 0; u < VL; ++u) v[u][c] = ((key + u >= j0 || key + u < keep) && key + u < visible) ? f[u] : 0.f;
                             }
                         }
                     }
@@ -550,7 +602,7 @@ __global__ __launch_bounds__(256) void attn_window_decode_kernel(
 #pragma unroll
                 for (int u = 0; u < VL; ++u) {
                     const int ku = key + u;
-                    if (ku < j0 || ku >= visible) continue;
+                    if ((ku < j0 && ku >= keep) || ku >= visible) continue;
                     const int pid = table[(size_t)b * max_blocks + ku / page];
                     if (pid < 0) continue;
 #pragma unroll
@@ -602,10 +654,11 @@ int aw_keys_a_block(int dk, int dv) {
 }
 
 // blocks of keys the window of a single token can touch when no request is longer than max_kv_len
-int aw_slots(int dk, int dv, int window, int max_kv_len) {
+int aw_slots(int dk, int dv, int window, int max_kv_len, int keep) {
     const int NK = AD_KEYS;
     const int span = window > 0 ? min(window, max_kv_len) : max_kv_len;
-    return (span + NK - 1) / NK + (window > 0 ? 1 : 0);      // a window may begin inside a block: one more
+    // a window may begin inside a block: one more; the blocks of the kept positions come first
+    return (span + NK - 1) / NK + (window > 0 ? 1 : 0) + (window > 0 ? (keep + NK - 1) / NK : 0);
 }
 
 }  // namespace
@@ -620,8 +673,9 @@ extern "C" int ri_rotate_kv_write(
         int H, int Hkv, int dk, int dv, int rot, const float* cos_t, const float* sin_t, int table_rows,
         const float* vcos, const float* vsin, int v_table_rows, int v_interleaved,
         const int* positions, const int* row_of_token, void* kc, void* vc, int num_pages,
-        const int* table, int max_blocks, int page, int write_kv, hipStream_t stream) {
+        const int* table, int max_blocks, int page, int write_kv, float unit_eps, hipStream_t stream) {
     RI_REQUIRE(T >= 0 && H > 0 && Hkv > 0 && dk > 0 && dv > 0 && page > 0, "ri_rotate_kv_write: bad sizes");
+    RI_REQUIRE(unit_eps >= 0.f && (unit_eps == 0.f || H + Hkv <= AW_NORM_HEADS), "ri_rotate_kv_write: unit queries and keys for up to %d heads", AW_NORM_HEADS);
     RI_REQUIRE(q_stride >= H * dk, "ri_rotate_kv_write: query row stride %d too small", q_stride);
     if (cos_t) RI_REQUIRE(rot > 0 && rot % 2 == 0 && rot <= dk && sin_t && table_rows > 0, "ri_rotate_kv_write: rot %d must be even and within the key size %d", rot, dk);
     if (vcos) RI_REQUIRE(dv % 2 == 0 && vsin && v_table_rows > 0, "ri_rotate_kv_write: a turned value needs an even size, got %d", dv);
@@ -630,9 +684,9 @@ extern "C" int ri_rotate_kv_write(
     if (T == 0) return 0;
     RI_REQUIRE(q && positions && row_of_token, "ri_rotate_kv_write: null pointer");
     if (dtype == RI_F32)
-        rotate_kv_write_kernel<float><<<T, 256, 0, stream>>>((float*)q, q_stride, (const float*)k, k_stride, (const float*)v, v_stride, H, Hkv, dk, dv, rot, cos_t, sin_t, vcos, vsin, v_interleaved, positions, row_of_token, (float*)kc, (float*)vc, table, max_blocks, page, write_kv);
+        rotate_kv_write_kernel<float><<<T, 256, 0, stream>>>((float*)q, q_stride, (const float*)k, k_stride, (const float*)v, v_stride, H, Hkv, dk, dv, rot, cos_t, sin_t, vcos, vsin, v_interleaved, positions, row_of_token, (float*)kc, (float*)vc, table, max_blocks, page, write_kv, unit_eps);
     else if (dtype == RI_BF16)
-        rotate_kv_write_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, Hkv, dk, dv, rot, cos_t, sin_t, vcos, vsin, v_interleaved, positions, row_of_token, (bf16_t*)kc, (bf16_t*)vc, table, max_blocks, page, write_kv);
+        rotate_kv_write_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, Hkv, dk, dv, rot, cos_t, sin_t, vcos, vsin, v_interleaved, positions, row_of_token, (bf16_t*)kc, (bf16_t*)vc, table, max_blocks, page, write_kv, unit_eps);
     else
         return ri_fail("ri_rotate_kv_write: unknown dtype %d", dtype);
     RI_LAUNCHED("ri_rotate_kv_write");
@@ -644,7 +698,7 @@ template <typename T>
 int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
               const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
               int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved,
-              int slots, float* workspace, const float* sink, hipStream_t stream) {
+              int slots, float* workspace, const float* sink, int keep, const float* sig_bias, hipStream_t stream) {
     const int G = H / Hkv, TQ = AW_ROWS / G;
     const int NK = aw_keys_a_block(dk, dv);
     const size_t lds = aw_lds_bytes(dk, dv, NK);
@@ -677,24 +731,25 @@ int aw_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, con
         RI_REQUIRE((long)Hkv * stretches <= 65535, "ri_attention_window: too many heads for the grid");
         part<<<dim3((slots + 3) / 4, Hkv * stretches, num_rows), 256, sizeof(float) * 4 * G * AD_KEYS, stream>>>(
             q, q_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, dk, dv, page, scale, window, slots, part_ml, part_o,
-            heads_a_wave);
+            heads_a_wave, keep, sig_bias);
         auto combine = NC == 1 ? attn_window_combine_kernel<T, 1> : NC == 2 ? attn_window_combine_kernel<T, 2>
                      : NC == 3 ? attn_window_combine_kernel<T, 3> : attn_window_combine_kernel<T, 4>;
         combine<<<dim3(H, num_rows), 64, 0, stream>>>(part_ml, part_o, out, out_stride, cu_q, q_start, kv_lens, H, dv, window, AD_KEYS, slots,
-                                                      vcos, vsin, v_interleaved, sink);
+                                                      vcos, vsin, v_interleaved, sink, keep, sig_bias != nullptr);
         return 0;
     }
     const int tiles = (Tn + TQ - 1) / TQ + num_rows;   // at most: every request may end in a short tile
     kernel<<<dim3(tiles, Hkv), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens,
-                                                   num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin, v_interleaved, sink);
+                                                   num_rows, H, Hkv, dk, dv, page, scale, window, TQ, NK, vcos, vsin, v_interleaved, sink,
+                                                   keep, sig_bias);
     return 0;
 }
 }  // namespace
 
 // Floats of workspace for a step of T single tokens whose longest request has max_kv_len keys
 // (0: such a step has one block of keys a row at most and needs none).
-extern "C" size_t ri_attention_window_workspace(int T, int H, int dk, int dv, int window, int max_kv_len) {
-    const int slots = aw_slots(dk, dv, window, max_kv_len);
+extern "C" size_t ri_attention_window_workspace(int T, int H, int dk, int dv, int window, int max_kv_len, int keep) {
+    const int slots = aw_slots(dk, dv, window, max_kv_len, window > 0 ? keep : 0);
     return slots <= 1 ? 0 : (size_t)T * H * slots * (dv + 2);
 }
 
@@ -704,13 +759,19 @@ extern "C" size_t ri_attention_window_workspace(int T, int H, int dk, int dv, in
 // single_tokens != 0: every row of the step has at most one token and row b's token is token
 // cu_q[b]; with a workspace of ri_attention_window_workspace floats the keys of a row are then
 // divided between blocks (the same bits as without).
+// keep: with a window, the first `keep` positions of a request stay in sight of every later query.
+// sig_bias [H] (null: softmax): the weight of a visible key is sigmoid(score + sig_bias[head]) and the
+// weights are not normalised over the keys (no sink then).
 extern "C" int ri_attention_window(
         const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kc, const void* vc,
         int num_pages, int page, int H, int Hkv, int dk, int dv, const int* table, int max_blocks,
         const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int T,
         float scale, int window, const float* vcos, const float* vsin, int v_table_rows, int v_interleaved,
-        int single_tokens, int max_kv_len, float* workspace, size_t workspace_floats, const float* sink, hipStream_t stream) {
+        int single_tokens, int max_kv_len, float* workspace, size_t workspace_floats, const float* sink,
+        int keep, const float* sig_bias, hipStream_t stream) {
     RI_REQUIRE(ri_attention_window_supported(H, Hkv, dk, dv), "ri_attention_window: sizes not taken (H=%d Hkv=%d dk=%d dv=%d)", H, Hkv, dk, dv);
+    RI_REQUIRE(keep >= 0 && !(sink && sig_bias), "ri_attention_window: keep must be >= 0, and sigmoid weights take no sink");
+    if (window == 0) keep = 0;
     RI_REQUIRE(T >= 0 && num_rows >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0 && page > 0, "ri_attention_window: bad sizes");
     RI_REQUIRE(q_stride >= H * dk && out_stride >= H * dv, "ri_attention_window: row strides too small");
     if (vcos) RI_REQUIRE(vsin && dv % 2 == 0 && v_table_rows > 0, "ri_attention_window: a turned value needs an even size and both tables");
@@ -719,16 +780,16 @@ extern "C" int ri_attention_window(
     RI_REQUIRE(Hkv <= 65535, "ri_attention_window: too many key/value heads for the grid");
     int slots = 0;
     if (single_tokens && workspace && max_kv_len > 0) {
-        slots = aw_slots(dk, dv, window, max_kv_len);
+        slots = aw_slots(dk, dv, window, max_kv_len, keep);
         if (slots <= 1) slots = 0;
         else RI_REQUIRE(workspace_floats >= (size_t)T * H * slots * (dv + 2) && slots <= 65535 && num_rows <= 65535 && H <= 65535,
                         "ri_attention_window: workspace of %zu floats for %d slots, or too many rows for the grid", workspace_floats, slots);
     }
     int rc;
     if (dtype == RI_F32)
-        rc = aw_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, sink, stream);
+        rc = aw_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, sink, keep, sig_bias, stream);
     else if (dtype == RI_BF16)
-        rc = aw_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, sink, stream);
+        rc = aw_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, slots, workspace, sink, keep, sig_bias, stream);
     else
         return ri_fail("ri_attention_window: unknown dtype %d", dtype);
     if (rc) return rc;
@@ -769,7 +830,8 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(
         const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int num_rows, int H, int Hkv, int dk, int dv, int page, float scale, int window,
-        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved, const float* __restrict__ sink) {
+        const float* __restrict__ vcos, const float* __restrict__ vsin, int v_interleaved, const float* __restrict__ sink,
+        int keep, const float* __restrict__ sig_bias) {
     extern __shared__ __align__(16) float lds[];
     constexpr int DKP = 8 * QU, KS = DKP + 4;
     const int vs_stride = dv + 8;
@@ -827,13 +889,15 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(
         for (int i = 0; i < 16; ++i) o[ft][i] = 0.f;
     float m = -INFINITY, l = 0.f;
 
-    for (int st = blk_first / AM_KEYS; st * AM_KEYS < blk_last; ++st) {
+    const float bias = sig_bias ? sig_bias[head] : 0.f;
+    for (int st = keep > 0 ? 0 : blk_first / AM_KEYS; st * AM_KEYS < blk_last; ++st) {
+        if (st * AM_KEYS >= keep && st < blk_first / AM_KEYS) st = blk_first / AM_KEYS;      // from the kept positions on to the window
         const int j_base = st * AM_KEYS;
         __syncthreads();                               // the last stage has been used (first pass: the zeros are written)
         if (tid < AM_KEYS) {
             const int j = j_base + tid;
             int off = -1;
-            if (j < blk_last && j >= blk_first) {
+            if (j < blk_last && (j >= blk_first || j < keep)) {
                 const int pid = table[(size_t)b * max_blocks + j / page];
                 if (pid >= 0) off = (pid * Hkv + g) * page + j % page;
             }
@@ -886,7 +950,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(
 #pragma unroll 1
         for (int half = 0; half < 2; ++half) {
             const int kt0 = j_base + 32 * half;        // first key of the tile
-            if (kt0 >= w_last || kt0 + 32 <= w_first) continue;     // none of the wave's queries sees it (the same for all lanes)
+            if (kt0 >= w_last || (kt0 + 32 <= w_first && kt0 >= keep)) continue;     // none of the wave's queries sees it (the same for all lanes)
             // S^T = K Q^T (the scale is in the query)
             aw_f16 s;
 #pragma unroll
@@ -906,26 +970,32 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int j = kt0 + 8 * (i >> 2) + 4 * lh + (i & 3);
-                const bool vis = row_on && j >= j_lo && j < j_hi;
+                const bool vis = row_on && (j >= j_lo || j < keep) && j < j_hi;
                 s[i] = vis ? s[i] : -INFINITY;
                 mt = fmaxf(mt, s[i]);
             }
-            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-            const float m_new = fmaxf(m, mt);
-            const bool any = m_new > -INFINITY;        // else the query has seen no key yet: nothing to add
-            const float alpha = any ? expf(m - m_new) : 1.f;
-            float psum = 0.f;
+            if (sig_bias) {
+                // sigmoids of the scores, added up as they are: nothing to rescale
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                s[i] = (any && s[i] > -INFINITY) ? expf(s[i] - m_new) : 0.f;
-                psum += s[i];
+                for (int i = 0; i < 16; ++i) s[i] = s[i] > -INFINITY ? 1.f / (1.f + expf(-(s[i] + bias))) : 0.f;
+            } else {
+                mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+                const float m_new = fmaxf(m, mt);
+                const bool any = m_new > -INFINITY;        // else the query has seen no key yet: nothing to add
+                const float alpha = any ? expf(m - m_new) : 1.f;
+                float psum = 0.f;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s[i] = (any && s[i] > -INFINITY) ? expf(s[i] - m_new) : 0.f;
+                    psum += s[i];
+                }
+                l = l * alpha + psum;
+                m = m_new;
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o[ft][i] *= alpha;
             }
-            l = l * alpha + psum;
-            m = m_new;
-#pragma unroll
-            for (int ft = 0; ft < FT; ++ft)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) o[ft][i] *= alpha;
             // O^T += V^T P^T
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
@@ -942,7 +1012,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(
     }
     // the sums of a query lie in the lane of its lower and of its upper half: add the two l
     l += __shfl_xor(l, 32, 64);
-    const float inv = aw_final_factor(m, l, sink, head);
+    const float inv = sig_bias ? 1.f : aw_final_factor(m, l, sink, head);
     __syncthreads();                                   // the last keys and values have been used
     float* ow = Os + (size_t)wave * 32 * dv;
     if (wave_on) {
@@ -977,7 +1047,8 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(
 template <typename T, int QU, int FT>
 int am_launch_as(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
                  const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
-                 int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, const float* sink, hipStream_t stream) {
+                 int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, const float* sink,
+                 int keep, const float* sig_bias, hipStream_t stream) {
     const int G = H / Hkv, HB = G < 4 ? G : 4, SB = 4 / HB, TQB = 32 * SB;
     const size_t lds = am_lds_bytes(QU, dv);
     auto kernel = attn_window_mfma_kernel<T, QU, FT>;
@@ -991,16 +1062,17 @@ int am_launch_as(const T* q, int q_stride, T* out, int out_stride, const T* kc, 
     }
     const int tiles = (Tn + TQB - 1) / TQB + num_rows;
     kernel<<<dim3(tiles, Hkv, (G + 3) / 4), 256, lds, stream>>>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start,
-                                                               kv_lens, num_rows, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink);
+                                                               kv_lens, num_rows, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, keep, sig_bias);
     return 0;
 }
 
 template <typename T>
 int am_launch(const T* q, int q_stride, T* out, int out_stride, const T* kc, const T* vc, const int* table, int max_blocks,
               const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int Tn, int H, int Hkv, int dk, int dv,
-              int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, const float* sink, hipStream_t stream) {
+              int page, float scale, int window, const float* vcos, const float* vsin, int v_interleaved, const float* sink,
+              int keep, const float* sig_bias, hipStream_t stream) {
 #define RI_AM(QU, FT) return am_launch_as<T, QU, FT>(q, q_stride, out, out_stride, kc, vc, table, max_blocks, cu_q, q_start, kv_lens, \
-        num_rows, Tn, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, stream)
+        num_rows, Tn, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, keep, sig_bias, stream)
     if (dk <= 64) { if (dv <= 64) RI_AM(8, 2); if (dv <= 128) RI_AM(8, 4); RI_AM(8, 8); }
     if (dk <= 128) { if (dv <= 64) RI_AM(16, 2); if (dv <= 128) RI_AM(16, 4); RI_AM(16, 8); }
     if (dv <= 64) RI_AM(32, 2);
@@ -1024,8 +1096,10 @@ extern "C" int ri_attention_window_mfma(
         int num_pages, int page, int H, int Hkv, int dk, int dv, const int* table, int max_blocks,
         const int* cu_q, const int* q_start, const int* kv_lens, int num_rows, int T,
         float scale, int window, const float* vcos, const float* vsin, int v_table_rows, int v_interleaved,
-        const float* sink, hipStream_t stream) {
+        const float* sink, int keep, const float* sig_bias, hipStream_t stream) {
     RI_REQUIRE(ri_attention_window_mfma_supported(H, Hkv, dk, dv), "ri_attention_window_mfma: sizes not taken (H=%d Hkv=%d dk=%d dv=%d)", H, Hkv, dk, dv);
+    RI_REQUIRE(keep >= 0 && !(sink && sig_bias), "ri_attention_window_mfma: keep must be >= 0, and sigmoid weights take no sink");
+    if (window == 0) keep = 0;
     RI_REQUIRE(T >= 0 && num_rows >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0 && page > 0, "ri_attention_window_mfma: bad sizes");
     RI_REQUIRE(q_stride >= H * dk && out_stride >= H * dv, "ri_attention_window_mfma: row strides too small");
     if (vcos) RI_REQUIRE(vsin && dv % 2 == 0 && v_table_rows > 0, "ri_attention_window_mfma: a turned value needs an even size and both tables");
@@ -1034,9 +1108,9 @@ extern "C" int ri_attention_window_mfma(
     RI_REQUIRE(Hkv <= 65535, "ri_attention_window_mfma: too many key/value heads for the grid");
     int rc;
     if (dtype == RI_F32)
-        rc = am_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, stream);
+        rc = am_launch<float>((const float*)q, q_stride, (float*)out, out_stride, (const float*)kc, (const float*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, keep, sig_bias, stream);
     else if (dtype == RI_BF16)
-        rc = am_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, stream);
+        rc = am_launch<bf16_t>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, num_rows, T, H, Hkv, dk, dv, page, scale, window, vcos, vsin, v_interleaved, sink, keep, sig_bias, stream);
     else
         return ri_fail("ri_attention_window_mfma: unknown dtype %d", dtype);
     if (rc) return rc;

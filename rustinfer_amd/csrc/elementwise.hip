@@ -57,12 +57,15 @@ extern "C" int ri_embed(const int* ids, const int* device_tokens, const void* ta
 template <typename TD, typename TW, typename TO, int BLOCK, int VEC, int PARTS>
 __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
         float* __restrict__ x, const TD* __restrict__ delta, int parts_rt, size_t part_stride,
-        const TW* __restrict__ w, TO* __restrict__ out, int d, float eps, const int* __restrict__ rows,
-        float* __restrict__ x_rows) {
+        const TW* __restrict__ w_all, TO* __restrict__ out, int d, float eps, const int* __restrict__ rows,
+        float* __restrict__ x_rows, int groups) {
     __shared__ float red[16];
     using L = VecLoad<VEC>;
+    // groups > 1: a row is `groups` consecutive parts of d values, each normed by itself: a block a part
     const int i_out = blockIdx.x;
-    const int r = rows ? rows[i_out] : i_out;
+    const int tok = groups > 1 ? i_out / groups : i_out, part = i_out - tok * groups;
+    const int r = (rows ? rows[tok] : tok) * groups + part;
+    const TW* w = w_all + (size_t)part * d;
     float* xr = x + (size_t)r * d;
     const TD* dr = delta ? delta + (size_t)r * d : nullptr;
     TO* o = out + (size_t)i_out * d;
@@ -152,8 +155,8 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
 
 template <typename TD, typename TW, typename TO>
 static int launch_add_rmsnorm(float* x, const void* delta, int parts, size_t part_stride, const void* w,
-                              void* out, int n_out, int d, float eps, const int* rows, float* x_rows, hipStream_t stream) {
-#define RI_NORM_ARGS x, (const TD*)delta, parts, part_stride, (const TW*)w, (TO*)out, d, eps, rows, x_rows
+                              void* out, int n_out, int d, float eps, const int* rows, float* x_rows, int groups, hipStream_t stream) {
+#define RI_NORM_ARGS x, (const TD*)delta, parts, part_stride, (const TW*)w, (TO*)out, d, eps, rows, x_rows, groups
 #define RI_NORM_LAUNCH(BLOCK, VEC) do { \
         if (parts == 1) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 1><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
         else if (parts == 2) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 2><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
@@ -179,9 +182,17 @@ static int launch_add_rmsnorm(float* x, const void* delta, int parts, size_t par
 // delta: null, or [parts][rows of x][d] of delta_dtype with part_stride elements between parts
 // rows: null, or the n_out rows of x to normalise (x itself is then left as it is); x_rows: null,
 // or where the sums x + delta of those rows go ([n_out][d], 32-bit)
+// groups > 1: every row is normed in that many equal consecutive parts, each by its own root mean square
+// (d, the row's width, must divide); the weight still has d entries.
 extern "C" int ri_add_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, long long part_stride,
                               const void* w, int w_dtype, void* out, int out_dtype, int n_out, int d,
-                              float eps, const int* rows, float* x_rows, hipStream_t stream) {
+                              float eps, const int* rows, float* x_rows, int groups, hipStream_t stream) {
+    RI_REQUIRE(groups >= 1 && d > 0 && d % groups == 0, "ri_add_rmsnorm: %d values do not split into %d equal parts", d, groups);
+    RI_REQUIRE((long long)n_out * groups <= 2147483647LL, "ri_add_rmsnorm: too many rows for the grid");
+    if (groups > 1) {
+        d /= groups;
+        n_out *= groups;
+    }
     RI_REQUIRE(!x_rows || rows, "ri_add_rmsnorm: x_rows goes with rows");
     RI_REQUIRE((uintptr_t)x_rows % 16 == 0, "ri_add_rmsnorm: operands must be 16-byte aligned");
     RI_REQUIRE(n_out >= 0 && d > 0, "ri_add_rmsnorm: bad sizes n_out=%d d=%d", n_out, d);
@@ -194,11 +205,12 @@ extern "C" int ri_add_rmsnorm(float* x, const void* delta, int delta_dtype, int 
     RI_REQUIRE(d % 4 != 0 || part_stride % 4 == 0, "ri_add_rmsnorm: part stride must be a multiple of 4");
     if (!delta) delta_dtype = out_dtype;
     const size_t ps = (size_t)part_stride;
-    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_F32) return launch_add_rmsnorm<float, float, float>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
-    if (delta_dtype == RI_BF16 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
-    if (delta_dtype == RI_BF16 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
-    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
-    if (delta_dtype == RI_F32 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
+    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_F32) return launch_add_rmsnorm<float, float, float>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, groups, stream);
+    if (delta_dtype == RI_BF16 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, groups, stream);
+    if (delta_dtype == RI_BF16 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, groups, stream);
+    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, groups, stream);
+    if (delta_dtype == RI_BF16 && w_dtype == RI_F32 && out_dtype == RI_F32) return launch_add_rmsnorm<bf16_t, float, float>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, groups, stream);
+    if (delta_dtype == RI_F32 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, groups, stream);
     return ri_fail("ri_add_rmsnorm: unsupported dtypes delta=%d weight=%d out=%d", delta_dtype, w_dtype, out_dtype);
 }
 

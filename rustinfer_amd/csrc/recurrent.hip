@@ -13,6 +13,14 @@
 //                is w = g, a u = beta g k, and beta k in place of k in the last term): q and k are made
 //                unit vectors (q also times q_scale), beta = sigmoid(bl_t), g = exp(-A softplus(gl_t +
 //                dt_bias)); several heads may share one head of q and k.
+//   channel-gated form: the gated form with a decay for every key channel, g = exp(-A_h softplus(gl + dt_bias))
+//                over heads x dk: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T is the walk with
+//                u-vector g * k, a u = beta k, w = g and beta k in the last term.
+//   channel-decay forms (no second term, a decay vector a token): S <- diag(w) S + k v^T, o = S^T r (+ skip_h v):
+//                w = sigmoid(gl + bias)^(1/tau) for every key channel and r times q_scale (gated linear
+//                attention); or w = exp(-A_h dt) for the whole head with dt = softplus(gl_h + dt_bias_h),
+//                k = dt B, r = C, several heads sharing one head of B and C, and the output also gets
+//                skip_h v (a state-space layer in its recurrent form).
 // Both terms of the delta form read the old state.  Everything after the projections is 32-bit.
 //
 // One kernel walks a request's tokens of the step in order; a step of single tokens is the same
@@ -52,6 +60,9 @@ struct ScanArgs {
     // w0 = A [H], ab = dt_bias [H]; kv_group heads share a head of r and k; r is multiplied by q_scale
     int gate_bf16, kv_group;
     float q_scale;
+    // the channel forms: al holds the decays' inputs ([T][>= H dk], or [T][>= H] for a decay a head) in the gates'
+    // dtype; ab their bias; w0 = A [H] where the form has one; decay_c = 1 / tau; skip [H] or null
+    const float* skip;
 };
 
 __device__ __forceinline__ float ld_gate(const void* p, size_t at, int is_bf16) {
@@ -99,13 +110,18 @@ __device__ __forceinline__ float wave_sum_rows(float x) {
            + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 48))));
 }
 
-template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT, bool GATED = false>
+// VAR: 0 the forms above; GATED and 1: the channel-gated form; not DELTA and 1: a decay a key channel
+// (sigmoid^(1/tau)); not DELTA and 2: a decay a head and token with k = dt B (the state-space form)
+template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT, bool GATED = false, int VAR = 0>
 __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) {
     static_assert(!GATED || (DELTA && !ROT), "the gated form is a delta form without a rotation");
+    static_assert(VAR == 0 || (!ROT && (GATED || !DELTA)), "the channel forms take no rotation");
+    constexpr bool VDEC = !DELTA && VAR > 0;            // a decay vector a token, no second term
+    constexpr bool CHAN_IN = (GATED && VAR == 1) || (VDEC && VAR == 1);    // decay inputs for every key channel, in the gates' dtype
     constexpr int SC_EPL = EPL;
     extern __shared__ __align__(16) float lds[];
     constexpr int TPW = SC_CH / NW;                    // tokens of a stretch a wave stages
-    constexpr int NA = DELTA ? 5 : 2;
+    constexpr int NA = DELTA ? 5 : (VDEC ? 3 : 2);
     const int P = a.P, DKP = P * R, dk = a.dk, dv = a.dv, H = a.H;
     const int CW = 64 / P, CPB = NW * CW;
     const int BUF = NA * SC_CH * DKP + SC_CH * CPB;    // floats of one of the two stretch buffers
@@ -124,15 +140,16 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
         const int i = pl * R + ii;
         S[ii] = (!fresh && col_ok && i < dk) ? Sg[(size_t)i * dv + j] : 0.f;
     }
-    const float dec = DELTA ? 0.f : a.decay[h];
+    const float dec = (DELTA || VDEC) ? 0.f : a.decay[h];
+    const float skip = (VDEC && a.skip) ? a.skip[h] : 0.f;
     const T* rp = (const T*)a.r; const T* kp = (const T*)a.k; const T* vp = (const T*)a.v;
     const T* wlp = (const T*)a.wl; const T* alp = (const T*)a.al;
 
     // what this thread stages of a stretch: asked for a stretch ahead, so that the walk hides the wait
-    float raw_r[TPW][SC_EPL], raw_k[TPW][SC_EPL], raw_w[DELTA && !GATED ? TPW : 1][SC_EPL], raw_a[DELTA && !GATED ? TPW : 1][SC_EPL];
+    float raw_r[TPW][SC_EPL], raw_k[TPW][SC_EPL], raw_w[(DELTA && !GATED) || CHAN_IN ? TPW : 1][SC_EPL], raw_a[DELTA && !GATED ? TPW : 1][SC_EPL];
     float raw_v[SC_CH];
-    float raw_gb[GATED ? TPW : 1], raw_ga[GATED ? TPW : 1];       // the gated form's two numbers a token
-    const int hk = GATED ? h / a.kv_group : h;                     // the head of r and k this head reads
+    float raw_gb[GATED ? TPW : 1], raw_ga[GATED || VAR == 2 ? TPW : 1];       // the gated forms' numbers a token and head
+    const int hk = (GATED || VAR == 2) ? h / a.kv_group : h;       // the head of r and k this head reads
     // ROT: the rotation partners of r and k (feature idx +- rot/2), asked for with them
     float part_r[ROT ? TPW : 1][SC_EPL], part_k[ROT ? TPW : 1][SC_EPL];
     const int rot_half = ROT ? a.rot >> 1 : 0;
@@ -160,11 +177,12 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                     raw_w[i][e] = on ? ld_f32(wlp + t * a.wl_stride + c) : 0.f;
                     raw_a[i][e] = on ? ld_f32(alp + t * a.al_stride + c) : 0.f;
                 }
+                if (CHAN_IN) raw_w[i][e] = on ? ld_gate(a.al, t * a.al_stride + h * dk + idx, a.gate_bf16) : 0.f;
             }
-            if (GATED) {
+            if (GATED || VAR == 2) {
                 const size_t t = (size_t)(t_lo + c0 + (tt < nc ? tt : 0));
-                raw_gb[i] = ld_gate(a.wl, t * a.wl_stride + h, a.gate_bf16);
-                raw_ga[i] = ld_gate(a.al, t * a.al_stride + h, a.gate_bf16);
+                if (GATED) raw_gb[i] = ld_gate(a.wl, t * a.wl_stride + h, a.gate_bf16);
+                if (!CHAN_IN) raw_ga[i] = ld_gate(a.al, t * a.al_stride + h, a.gate_bf16);
             }
         }
 #pragma unroll
@@ -180,13 +198,55 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
         float* ks = rs + SC_CH * DKP;
         float* us = ks + SC_CH * DKP;                  // the delta form's three
         float* aus = us + SC_CH * DKP;
-        float* ws = aus + SC_CH * DKP;
+        float* ws = VDEC ? us : aus + SC_CH * DKP;     // (the channel-decay forms keep r, k and w only)
         float* vs = buf + NA * SC_CH * DKP;            // [SC_CH][CPB]
 #pragma unroll
         for (int i = 0; i < TPW; ++i) {
             const int tt = wave + i * NW;
             if (tt >= nc) continue;
-            if (GATED) {
+            if (VDEC) {
+                float dt = 0.f, dec = 0.f;
+                if (VAR == 2) {
+                    dt = softplusf_(raw_ga[i] + a.ab[h]);
+                    dec = expf(-a.w0[h] * dt);
+                }
+#pragma unroll
+                for (int e = 0; e < SC_EPL; ++e) {
+                    const int idx = e * 64 + lane;
+                    if (idx >= DKP) continue;
+                    float r = 0.f, k = 0.f, w = 0.f;
+                    if (idx < dk) {
+                        if (VAR == 1) {
+                            // sigmoid(z)^(1/tau) = exp(-softplus(-z) / tau)
+                            r = raw_r[i][e] * a.q_scale; k = raw_k[i][e];
+                            w = expf(-softplusf_(-(raw_w[i][e] + a.ab[h * dk + idx])) * a.decay_c);
+                        } else {
+                            r = raw_r[i][e]; k = dt * raw_k[i][e]; w = dec;
+                        }
+                    }
+                    rs[tt * DKP + idx] = r; ks[tt * DKP + idx] = k; ws[tt * DKP + idx] = w;
+                }
+            } else if (GATED && VAR == 1) {
+                float sk = 0.f, sq = 0.f;
+#pragma unroll
+                for (int e = 0; e < SC_EPL; ++e) { sk = fmaf(raw_k[i][e], raw_k[i][e], sk); sq = fmaf(raw_r[i][e], raw_r[i][e], sq); }
+                sk = wave_sum_rows(sk);
+                sq = wave_sum_rows(sq);
+                const float inv_k = 1.f / sqrtf(sk + a.unit_eps), inv_q = a.q_scale / sqrtf(sq + a.unit_eps);
+                const float beta = 1.f / (1.f + expf(-raw_gb[i]));
+                const float rate = a.w0[h];
+#pragma unroll
+                for (int e = 0; e < SC_EPL; ++e) {
+                    const int idx = e * 64 + lane;
+                    if (idx >= DKP) continue;
+                    const bool in = idx < dk;
+                    const float u = in ? raw_k[i][e] * inv_k : 0.f;
+                    const float g = in ? expf(-rate * softplusf_(raw_w[i][e] + a.ab[h * dk + idx])) : 0.f;
+                    rs[tt * DKP + idx] = in ? raw_r[i][e] * inv_q : 0.f;
+                    us[tt * DKP + idx] = g * u; ks[tt * DKP + idx] = beta * u;
+                    aus[tt * DKP + idx] = beta * u; ws[tt * DKP + idx] = g;
+                }
+            } else if (GATED) {
                 float sk = 0.f, sq = 0.f;
 #pragma unroll
                 for (int e = 0; e < SC_EPL; ++e) { sk = fmaf(raw_k[i][e], raw_k[i][e], sk); sq = fmaf(raw_r[i][e], raw_r[i][e], sq); }
@@ -265,7 +325,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
         const float* ks = rs + SC_CH * DKP;
         const float* us = ks + SC_CH * DKP;
         const float* aus = us + SC_CH * DKP;
-        const float* ws = aus + SC_CH * DKP;
+        const float* ws = VDEC ? us : aus + SC_CH * DKP;
         const float* vs = buf + NA * SC_CH * DKP;
 #pragma unroll 4
         for (int tt = 0; tt < nc; ++tt) {
@@ -290,6 +350,14 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                     S[ii + 2] = fmaf(w4.z, S[ii + 2], fmaf(-a4.z, dot, k4.z * vv));
                     S[ii + 3] = fmaf(w4.w, S[ii + 3], fmaf(-a4.w, dot, k4.w * vv));
                 }
+            } else if (VDEC) {
+#pragma unroll
+                for (int ii = 0; ii < R; ii += 4) {
+                    const float4 w4 = *reinterpret_cast<const float4*>(ws + base + ii);
+                    const float4 k4 = *reinterpret_cast<const float4*>(ks + base + ii);
+                    S[ii] = fmaf(w4.x, S[ii], k4.x * vv); S[ii + 1] = fmaf(w4.y, S[ii + 1], k4.y * vv);
+                    S[ii + 2] = fmaf(w4.z, S[ii + 2], k4.z * vv); S[ii + 3] = fmaf(w4.w, S[ii + 3], k4.w * vv);
+                }
             } else {
 #pragma unroll
                 for (int ii = 0; ii < R; ii += 4) {
@@ -306,6 +374,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                 o = fmaf(r4.z, S[ii + 2], o); o = fmaf(r4.w, S[ii + 3], o);
             }
             o = group_sum(o, P);
+            if (VDEC) o = fmaf(skip, vv, o);
             if (pl == 0 && col_ok) a.out[(size_t)(t_lo + c0 + tt) * a.out_stride + h * dv + j] = o;
         }
     }
@@ -316,12 +385,12 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
     }
 }
 
-template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT, bool GATED = false>
+template <typename T, bool DELTA, int R, int NW, int EPL, bool ROT, bool GATED = false, int VAR = 0>
 int launch_scan_rot(const ScanArgs& a, int num_rows, hipStream_t stream) {
     const int P = a.P, DKP = P * R, CPB = NW * (64 / P);
-    const size_t lds = sizeof(float) * 2 * ((DELTA ? 5 : 2) * SC_CH * DKP + SC_CH * CPB);
+    const size_t lds = sizeof(float) * 2 * ((DELTA ? 5 : (VAR > 0 ? 3 : 2)) * SC_CH * DKP + SC_CH * CPB);
     dim3 grid((a.dv + CPB - 1) / CPB, a.H, num_rows);
-    auto kernel = linear_scan_kernel<T, DELTA, R, NW, EPL, ROT, GATED>;
+    auto kernel = linear_scan_kernel<T, DELTA, R, NW, EPL, ROT, GATED, VAR>;
     if (lds > 64 * 1024) {
         // more LDS than a kernel gets unasked (the delta form with more than 128 key rows)
         static bool asked = false;
@@ -335,29 +404,30 @@ int launch_scan_rot(const ScanArgs& a, int num_rows, hipStream_t stream) {
     return 0;
 }
 
-template <typename T, bool DELTA, int R, int NW, int EPL, bool GATED = false>
+template <typename T, bool DELTA, int R, int NW, int EPL, bool GATED = false, int VAR = 0>
 int launch_scan_as(const ScanArgs& a, int num_rows, hipStream_t stream) {
-    if constexpr (GATED) return launch_scan_rot<T, true, R, NW, EPL, false, true>(a, num_rows, stream);
+    if constexpr (GATED) return launch_scan_rot<T, true, R, NW, EPL, false, true, VAR>(a, num_rows, stream);
+    if constexpr (VAR > 0) return launch_scan_rot<T, false, R, NW, EPL, false, false, VAR>(a, num_rows, stream);
     if constexpr (!DELTA) {
         if (a.rot_cos != nullptr || a.k_scale != 1.f) return launch_scan_rot<T, DELTA, R, NW, EPL, true>(a, num_rows, stream);
     }
     return launch_scan_rot<T, DELTA, R, NW, EPL, false>(a, num_rows, stream);
 }
 
-template <typename T, bool DELTA, int R, bool GATED = false>
+template <typename T, bool DELTA, int R, bool GATED = false, int VAR = 0>
 int launch_scan(const ScanArgs& a, int num_rows, hipStream_t stream) {
     // Four waves a block share the staging of a stretch (a wave alone spends more instructions on
     // staging than on the walk); one wave where a head has no more than 64 threads.
     const bool four = (long)a.dv * a.P > 64;
     const int epl = (a.dk + 63) / 64;
     if (four) {
-        if (epl == 1) return launch_scan_as<T, DELTA, R, 4, 1, GATED>(a, num_rows, stream);
-        if (epl == 2) return launch_scan_as<T, DELTA, R, 4, 2, GATED>(a, num_rows, stream);
-        return launch_scan_as<T, DELTA, R, 4, 4, GATED>(a, num_rows, stream);
+        if (epl == 1) return launch_scan_as<T, DELTA, R, 4, 1, GATED, VAR>(a, num_rows, stream);
+        if (epl == 2) return launch_scan_as<T, DELTA, R, 4, 2, GATED, VAR>(a, num_rows, stream);
+        return launch_scan_as<T, DELTA, R, 4, 4, GATED, VAR>(a, num_rows, stream);
     }
-    if (epl == 1) return launch_scan_as<T, DELTA, R, 1, 1, GATED>(a, num_rows, stream);
-    if (epl == 2) return launch_scan_as<T, DELTA, R, 1, 2, GATED>(a, num_rows, stream);
-    return launch_scan_as<T, DELTA, R, 1, 4, GATED>(a, num_rows, stream);
+    if (epl == 1) return launch_scan_as<T, DELTA, R, 1, 1, GATED, VAR>(a, num_rows, stream);
+    if (epl == 2) return launch_scan_as<T, DELTA, R, 1, 2, GATED, VAR>(a, num_rows, stream);
+    return launch_scan_as<T, DELTA, R, 1, 4, GATED, VAR>(a, num_rows, stream);
 }
 
 }  // namespace
@@ -397,7 +467,7 @@ extern "C" int ri_linear_scan(
     a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
     a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = silu_in; a.unit_eps = unit_eps; a.decay_c = decay_c;
     a.rot_cos = rot_cos; a.rot_sin = rot_sin; a.rot = rot_cos ? rot : 0; a.k_scale = k_scale;
-    a.gate_bf16 = 0; a.kv_group = 1; a.q_scale = 1.f;
+    a.gate_bf16 = 0; a.kv_group = 1; a.q_scale = 1.f; a.skip = nullptr;
     int rc;
 #define RI_SCAN(TT, DD) (R == 8 ? launch_scan<TT, DD, 8>(a, num_rows, stream) : launch_scan<TT, DD, 16>(a, num_rows, stream))
     if (dtype == RI_F32) rc = delta ? RI_SCAN(float, true) : RI_SCAN(float, false);
@@ -438,10 +508,88 @@ extern "C" int ri_gated_delta_scan(
     a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
     a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = 0; a.unit_eps = unit_eps; a.decay_c = 0.f;
     a.rot_cos = nullptr; a.rot_sin = nullptr; a.rot = 0; a.k_scale = 1.f;
-    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale;
+    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale; a.skip = nullptr;
     const int rc = R == 8 ? launch_scan<float, true, 8, true>(a, num_rows, stream) : launch_scan<float, true, 16, true>(a, num_rows, stream);
     if (rc) return rc;
     RI_LAUNCHED("ri_gated_delta_scan");
+    return 0;
+}
+
+// The channel-gated form of the walk: ri_gated_delta_scan with a decay for every key channel.  gl [T, >= H dk]
+// holds the decays' inputs in gate_dtype (as bl [T, >= H]), dt_bias [H dk] and A [H] are 32-bit:
+// g = exp(-A_h softplus(gl + dt_bias)) over heads x dk.
+extern "C" int ri_channel_delta_scan(
+        const float* q, int q_stride, const float* k, int k_stride, const float* v, int v_stride,
+        const void* bl, int bl_stride, const void* gl, int gl_stride, int gate_dtype,
+        const float* A, const float* dt_bias, float unit_eps, float q_scale,
+        float* state, int num_slots, float* out, int out_stride,
+        const int* cu_q, const int* q_start, const int* slots, int num_rows, int T,
+        int H, int Hk, int dk, int dv, hipStream_t stream) {
+    RI_REQUIRE(H > 0 && Hk > 0 && H % Hk == 0 && dk > 0 && dv > 0 && dk <= 256, "ri_channel_delta_scan: bad sizes H=%d Hk=%d dk=%d dv=%d (dk <= 256)", H, Hk, dk, dv);
+    RI_REQUIRE(num_rows >= 0 && T >= 0 && num_slots > 0, "ri_channel_delta_scan: bad counts");
+    RI_REQUIRE(q_stride >= Hk * dk && k_stride >= Hk * dk && v_stride >= H * dv && out_stride >= H * dv && bl_stride >= H && gl_stride >= H * dk,
+               "ri_channel_delta_scan: row strides too small");
+    RI_REQUIRE(gate_dtype == RI_F32 || gate_dtype == RI_BF16, "ri_channel_delta_scan: unknown dtype %d", gate_dtype);
+    if (num_rows == 0 || T == 0) return 0;
+    RI_REQUIRE(q && k && v && bl && gl && A && dt_bias && state && out && cu_q && q_start && slots, "ri_channel_delta_scan: null pointer");
+    RI_REQUIRE(H <= 65535 && num_rows <= 65535, "ri_channel_delta_scan: too many heads or rows for the grid");
+    const int R = dk <= 128 ? 8 : 16;
+    int P = 1;
+    while (P * R < dk) P *= 2;
+    ScanArgs a;
+    a.r = q; a.k = k; a.v = v; a.wl = bl; a.al = gl;
+    a.r_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.wl_stride = bl_stride; a.al_stride = gl_stride;
+    a.w0 = A; a.ab = dt_bias; a.decay = nullptr; a.state = state; a.out = out; a.out_stride = out_stride;
+    a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
+    a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = 0; a.unit_eps = unit_eps; a.decay_c = 0.f;
+    a.rot_cos = nullptr; a.rot_sin = nullptr; a.rot = 0; a.k_scale = 1.f;
+    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale; a.skip = nullptr;
+    const int rc = R == 8 ? launch_scan<float, true, 8, true, 1>(a, num_rows, stream) : launch_scan<float, true, 16, true, 1>(a, num_rows, stream);
+    if (rc) return rc;
+    RI_LAUNCHED("ri_channel_delta_scan");
+    return 0;
+}
+
+// The channel-decay forms of the walk: S <- diag(w) S + k v^T, out = S^T r (+ skip_h v).
+//   mode 1: r, k [T, >= H dk], v [T, >= H dv] in `dtype`; gl [T, >= H dk] in gate_dtype, bias [H dk]:
+//           w = sigmoid(gl + bias)^(1 / tau) for every key channel, r times q_scale.
+//   mode 2: r, k [T, >= Hk dk] (head h reads head h / (H / Hk)), v [T, >= H dv] in `dtype`; gl [T, >= H] in
+//           gate_dtype, bias [H], A [H]: dt = softplus(gl + bias), w = exp(-A dt) for the whole head, k times dt.
+// skip [H] or null.  state [slots][H][dk][dv] and out are 32-bit; a row whose q_start is 0 starts from zeros.
+extern "C" int ri_decay_scan(
+        int mode, const void* r, int r_stride, const void* k, int k_stride, const void* v, int v_stride, int dtype,
+        const void* gl, int gl_stride, int gate_dtype, const float* bias, const float* A, float inv_tau, float q_scale,
+        const float* skip, float* state, int num_slots, float* out, int out_stride,
+        const int* cu_q, const int* q_start, const int* slots, int num_rows, int T,
+        int H, int Hk, int dk, int dv, hipStream_t stream) {
+    RI_REQUIRE(mode == 1 || mode == 2, "ri_decay_scan: mode %d", mode);
+    RI_REQUIRE(H > 0 && Hk > 0 && H % Hk == 0 && dk > 0 && dv > 0 && dk <= 256, "ri_decay_scan: bad sizes H=%d Hk=%d dk=%d dv=%d (dk <= 256)", H, Hk, dk, dv);
+    RI_REQUIRE(mode == 2 || Hk == H, "ri_decay_scan: a decay a key channel goes with a head of r and k for every head");
+    RI_REQUIRE(num_rows >= 0 && T >= 0 && num_slots > 0, "ri_decay_scan: bad counts");
+    RI_REQUIRE(r_stride >= Hk * dk && k_stride >= Hk * dk && v_stride >= H * dv && out_stride >= H * dv && gl_stride >= (mode == 1 ? H * dk : H),
+               "ri_decay_scan: row strides too small");
+    RI_REQUIRE((dtype == RI_F32 || dtype == RI_BF16) && (gate_dtype == RI_F32 || gate_dtype == RI_BF16), "ri_decay_scan: unknown dtype");
+    if (num_rows == 0 || T == 0) return 0;
+    RI_REQUIRE(r && k && v && gl && bias && (mode == 1 || A) && state && out && cu_q && q_start && slots, "ri_decay_scan: null pointer");
+    RI_REQUIRE(H <= 65535 && num_rows <= 65535, "ri_decay_scan: too many heads or rows for the grid");
+    const int R = dk <= 128 ? 8 : 16;
+    int P = 1;
+    while (P * R < dk) P *= 2;
+    ScanArgs a;
+    a.r = r; a.k = k; a.v = v; a.wl = nullptr; a.al = gl;
+    a.r_stride = r_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.wl_stride = 0; a.al_stride = gl_stride;
+    a.w0 = A; a.ab = bias; a.decay = nullptr; a.state = state; a.out = out; a.out_stride = out_stride;
+    a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
+    a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = 0; a.unit_eps = 0.f; a.decay_c = inv_tau;
+    a.rot_cos = nullptr; a.rot_sin = nullptr; a.rot = 0; a.k_scale = 1.f;
+    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale; a.skip = skip;
+    int rc;
+#define RI_DSCAN(TT, VV) (R == 8 ? launch_scan<TT, false, 8, false, VV>(a, num_rows, stream) : launch_scan<TT, false, 16, false, VV>(a, num_rows, stream))
+    if (dtype == RI_F32) rc = mode == 1 ? RI_DSCAN(float, 1) : RI_DSCAN(float, 2);
+    else rc = mode == 1 ? RI_DSCAN(bf16_t, 1) : RI_DSCAN(bf16_t, 2);
+#undef RI_DSCAN
+    if (rc) return rc;
+    RI_LAUNCHED("ri_decay_scan");
     return 0;
 }
 
@@ -449,6 +597,7 @@ extern "C" int ri_gated_delta_scan(
 // y = o / sqrt(mean_group(o^2) + eps) * w * sigmoid(gate) (w null: no weight; gate_silu: silu(gate)
 // in place of the sigmoid): the norm over groups of `group`
 // consecutive features (all of a row, or a head) that follows the walk, with the output gate.
+// gate_first: the gate multiplies o before the norm (the norm is over o * silu(gate)).
 // o is 32-bit; gate and out are activations of `dtype` with row strides; w has n entries.
 // A wave a group, or the whole block for a group of more than 512 features.
 // ---------------------------------------------------------------------------
@@ -458,7 +607,7 @@ namespace {
 template <typename T, typename TW, bool BLOCK_GROUP>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(
         const float* __restrict__ o, int o_stride, int n, int group, const TW* __restrict__ w,
-        const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride, float eps, int gate_silu) {
+        const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride, float eps, int gate_silu, int gate_first) {
     __shared__ float red[16];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const float* orow = o + (size_t)t * o_stride;
@@ -467,14 +616,19 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
     if (g0 >= n) return;
     const int first = BLOCK_GROUP ? threadIdx.x : lane, step = BLOCK_GROUP ? blockDim.x : 64;
     float ss = 0.f;
-    for (int i = first; i < group; i += step) { const float x = orow[g0 + i]; ss = fmaf(x, x, ss); }
+    const bool pre = gate_first && gate;
+    auto gated = [&](int c) -> float {
+        const float z = ld_f32(gate + (size_t)t * gate_stride + c);
+        return orow[c] * (gate_silu ? siluf_(z) : sigmoidf_(z));
+    };
+    for (int i = first; i < group; i += step) { const float x = pre ? gated(g0 + i) : orow[g0 + i]; ss = fmaf(x, x, ss); }
     ss = BLOCK_GROUP ? block_sum(ss, red) : wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)group + eps);
     for (int i = first; i < group; i += step) {
         const int c = g0 + i;
-        float y = orow[c] * inv;
+        float y = (pre ? gated(c) : orow[c]) * inv;
         if (w) y *= ld_f32(w + c);
-        if (gate) {
+        if (gate && !pre) {
             const float z = ld_f32(gate + (size_t)t * gate_stride + c);
             y *= gate_silu ? siluf_(z) : sigmoidf_(z);
         }
@@ -485,7 +639,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
 
 extern "C" int ri_gated_group_norm(const float* o, int o_stride, int T, int n, int group, const void* w, int w_dtype,
                                    const void* gate, int gate_stride, void* out, int out_stride, int dtype,
-                                   float eps, int gate_silu, hipStream_t stream) {
+                                   float eps, int gate_silu, int gate_first, hipStream_t stream) {
     RI_REQUIRE(T >= 0 && n > 0 && group > 0 && n % group == 0, "ri_gated_group_norm: %d features do not split into groups of %d", n, group);
     RI_REQUIRE(o_stride >= n && out_stride >= n && (!gate || gate_stride >= n), "ri_gated_group_norm: row strides too small");
     if (T == 0) return 0;
@@ -496,8 +650,8 @@ extern "C" int ri_gated_group_norm(const float* o, int o_stride, int T, int n, i
     const bool big = group > 512;
     const int block = big ? 256 : 64 * min(4, groups);
     const dim3 grid(T, big ? groups : (groups + block / 64 - 1) / (block / 64));
-#define RI_GGN(TT, TW) do { if (big) gated_group_norm_kernel<TT, TW, true><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps, gate_silu); \
-        else gated_group_norm_kernel<TT, TW, false><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps, gate_silu); } while (0)
+#define RI_GGN(TT, TW) do { if (big) gated_group_norm_kernel<TT, TW, true><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps, gate_silu, gate_first); \
+        else gated_group_norm_kernel<TT, TW, false><<<grid, block, 0, stream>>>(o, o_stride, n, group, (const TW*)w, (const TT*)gate, gate_stride, (TT*)out, out_stride, eps, gate_silu, gate_first); } while (0)
     if (dtype == RI_F32 && w_dtype == RI_F32) RI_GGN(float, float);
     else if (dtype == RI_BF16 && w_dtype == RI_F32) RI_GGN(bf16_t, float);
     else if (dtype == RI_BF16 && w_dtype == RI_BF16) RI_GGN(bf16_t, bf16_t);

@@ -1,7 +1,7 @@
 // A short causal convolution over time, channel by channel, with the inputs of the last taps - 1
 // positions carried from step to step:
 //
-//   y[p][c] = f( sum_j w[c][j] * x[p - (taps - 1) + j][c] ),   j = 0 .. taps - 1,   x = 0 before position 0
+//   y[p][c] = f( sum_j w[c][j] * x[p - (taps - 1) + j][c] + bias[c] ),   j = 0 .. taps - 1,   x = 0 before position 0
 //
 // (the last column of w multiplies the current token's input), f = silu or nothing.  Up to four
 // segments of channels (the columns of several projections) go through one launch; each has its input
@@ -25,6 +25,7 @@ constexpr int SC_MAX_TAPS = 8;
 struct ConvSeg {
     const void* x;       // [T][x_stride], the segment's first column
     const void* w;       // [n][taps]
+    const float* bias;   // [n] or null
     int x_stride, n, out_col, first_block;
 };
 
@@ -55,6 +56,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const ConvArgs a) {
     float w[SC_MAX_TAPS];
 #pragma unroll
     for (int j = 0; j < SC_MAX_TAPS; ++j) w[j] = j < taps ? ld_f32(reinterpret_cast<const T*>(sg.w) + (size_t)c * taps + j) : 0.f;
+    const float bias = sg.bias ? sg.bias[c] : 0.f;
     // the input at the row's local index i (negative: before this step)
     auto input = [&](int i) -> float {
         if (i >= 0) return ld_f32(xs + (size_t)(t_lo + i) * sg.x_stride);
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const ConvArgs a) {
             const int i = i8 + u;
             if (i >= i1) break;
             const float cur = ahead[u];
-            float y = 0.f;
+            float y = bias;
 #pragma unroll
             for (int j = 0; j < SC_MAX_TAPS - 1; ++j) if (j < hist) y = fmaf(w[j], win[j], y);
             y = fmaf(w[hist], cur, y);
@@ -115,7 +117,8 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const ConvArgs a) {
 
 // nseg segments: x[s] (columns of `dtype`, row stride x_stride[s]), w[s] [n[s]][taps] of `dtype`; the
 // segments' outputs lie side by side in out [T][out_stride] (32-bit) and in state, in the order given.
-extern "C" int ri_short_conv(int nseg, const void* const* x, const int* x_stride, const void* const* w, const int* n,
+// bias: null, or nseg pointers to 32-bit [n[s]] (each may be null).
+extern "C" int ri_short_conv(int nseg, const void* const* x, const int* x_stride, const void* const* w, const float* const* bias, const int* n,
                              int dtype, int taps, int silu, float* state, int num_slots, float* out, int out_stride,
                              const int* cu_q, const int* q_start, const int* slots, int num_rows, int T, int max_q_len,
                              hipStream_t stream) {
@@ -127,6 +130,7 @@ extern "C" int ri_short_conv(int nseg, const void* const* x, const int* x_stride
     for (int s = 0; s < nseg; ++s) {
         RI_REQUIRE(n[s] > 0 && x_stride[s] >= n[s], "ri_short_conv: segment %d: bad sizes", s);
         a.seg[s].x = x[s]; a.seg[s].w = w[s]; a.seg[s].x_stride = x_stride[s]; a.seg[s].n = n[s];
+        a.seg[s].bias = bias ? bias[s] : nullptr;
         a.seg[s].out_col = C; a.seg[s].first_block = blocks;
         C += n[s];
         blocks += (n[s] + 255) / 256;

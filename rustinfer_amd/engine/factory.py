@@ -42,9 +42,9 @@ def pages_that_fit(needs, page_size: int, element_size: int, free_bytes: int, me
     ``max_requests`` requests (and the scratch slot) has been taken from it; at most what
     ``max_requests`` full-length requests can use.  ``needs``: what ``DecoderModel.cache_needs``
     returns (serve_loop.rs:391-501)."""
-    from ..parts.base import PagedKVNeed, StateNeed
+    from ..parts.base import PagedKVNeed, StateNeed, simple_needs
     per_page = state = 0
-    for need in needs.values():
+    for need in (n for whole in needs.values() for n in simple_needs(whole)):
         if isinstance(need, PagedKVNeed):
             per_page += need.num_kv_heads * (need.head_dim + need.value_dim) * page_size * element_size
         elif isinstance(need, StateNeed):
@@ -79,7 +79,7 @@ def second_copy_budget(model, rt: Runtime, page_size: int, num_pages: int, max_r
     else the share ``reserve`` of the device's memory) and a margin.  None off a GPU."""
     if rt.device.type != "cuda" or not torch.cuda.is_available():
         return None
-    from ..parts.base import PagedKVNeed
+    from ..parts.base import PagedKVNeed, simple_needs
     el = 2 if rt.dtype == torch.bfloat16 else 4
     weights = 0
     for spec in model.param_specs().values():
@@ -92,7 +92,7 @@ def second_copy_budget(model, rt: Runtime, page_size: int, num_pages: int, max_r
     free += max(0, torch.cuda.memory_reserved(rt.device) - torch.cuda.memory_allocated(rt.device))
     if num_pages > 0:
         cache = sum(need.num_kv_heads * (need.head_dim + need.value_dim) * page_size * el * (num_pages + 1)
-                    for need in model.cache_needs().values() if isinstance(need, PagedKVNeed))
+                    for whole in model.cache_needs().values() for need in simple_needs(whole) if isinstance(need, PagedKVNeed))
     else:
         cache = int(reserve * total)
     return max(0, free - weights - cache - TILE_MARGIN_BYTES)

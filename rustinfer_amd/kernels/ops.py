@@ -154,8 +154,10 @@ def norm_residual(x: torch.Tensor, delta: Optional[torch.Tensor], weight: Option
 
 def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                 out: torch.Tensor, rows: Optional[torch.Tensor] = None,
-                x_rows: Optional[torch.Tensor] = None) -> None:
-    """``x += delta`` (32-bit residual, in place unless ``rows`` gathers), ``out = rmsnorm(x) * weight``.
+                x_rows: Optional[torch.Tensor] = None, groups: int = 1) -> None:
+    """``groups > 1``: every row is normed in that many equal consecutive parts, each divided by its own
+    root mean square.  ``out`` may be 32-bit whatever the delta's dtype (a consumer that rounds later).
+    ``x += delta`` (32-bit residual, in place unless ``rows`` gathers), ``out = rmsnorm(x) * weight``.
     ``delta`` is ``[T, d]`` in the activations' dtype or 32-bit, or a stack ``[P, T, d]`` of 32-bit
     partial sums that are added up here.  With ``rows``, ``x_rows`` ([len(rows), d], 32-bit) takes
     the sums ``x + delta`` of those rows: the residual stream cut down to them."""
@@ -175,17 +177,19 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         if tuple(delta.shape[-2:]) != (T, d) or delta.stride(-1) != 1 or delta.stride(-2) != d \
                 or (delta.dim() == 3 and delta.dtype != torch.float32) or delta.dim() not in (2, 3):
             raise KernelError("add_rmsnorm: delta must be [T, d] or a float32 stack [P, T, d] with contiguous rows")
-        if delta.dtype not in (out.dtype, torch.float32):
+        if delta.dtype not in (out.dtype, torch.float32) and out.dtype != torch.float32:
             raise KernelError("add_rmsnorm: delta must be in the dtype of out or float32")
         ddt = _dt(delta)
     if weight.numel() != d or not weight.is_contiguous():
         raise KernelError(f"add_rmsnorm: weight must have {d} entries")
+    if groups < 1 or d % groups:
+        raise KernelError(f"add_rmsnorm: {d} values do not split into {groups} equal parts")
     if x_rows is not None and (rows is None or tuple(x_rows.shape) != (n_out, d) or x_rows.dtype != torch.float32
                                or not x_rows.is_contiguous()):
         raise KernelError(f"add_rmsnorm: x_rows goes with rows and must be contiguous float32 [{n_out}, {d}]")
     _check(_lib().ri_add_rmsnorm(_ptr(x), _ptr(delta), ddt, parts, ctypes.c_longlong(stride), _ptr(weight),
                                  _dt(weight), _ptr(out), _dt(out), n_out, d, ctypes.c_float(eps),
-                                 _ptr(rows), _ptr(x_rows), _stream()))
+                                 _ptr(rows), _ptr(x_rows), int(groups), _stream()))
 
 
 def _check_cache(k_cache, v_cache, Hkv, hd, page, act_dtype, name):
@@ -900,8 +904,10 @@ def _check_cache_kv(k_cache, v_cache, Hkv, dk, dv, page, act_dtype, name):
 def rotate_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], H: int, Hkv: int,
                     dk: int, dv: int, rotary, value_rotary, positions: torch.Tensor, row_of_token: torch.Tensor,
                     k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, page: int,
-                    write_kv: bool = True, interleaved_values: bool = False) -> None:
-    """Rotate ``q [T, H dk]`` in place (``rotary = (cos, sin, rot_dim)``: the first ``rot_dim``
+                    write_kv: bool = True, interleaved_values: bool = False, unit_eps: float = 0.0) -> None:
+    """``unit_eps > 0``: every head of q and k is also divided by ``sqrt(mean(.^2) + unit_eps)`` (a rotation
+    leaves that mean as it is, so it does not matter on which side of it the division stands).
+    Rotate ``q [T, H dk]`` in place (``rotary = (cos, sin, rot_dim)``: the first ``rot_dim``
     features of a head, feature i with i + rot_dim/2) and write this step's keys (rotated the same
     way) and values into their pages.  ``value_rotary = (cos, sin)`` ``[positions, dv/2]``: a value
     is cached turned by its position over all its features, pair m = (m, m + dv/2), or
@@ -935,7 +941,7 @@ def rotate_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torc
         _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache),
         k_cache.shape[0] if k_cache is not None else 0, _ptr(block_table),
         block_table.shape[1] if block_table is not None and block_table.dim() == 2 else 0, page,
-        int(bool(write_kv)), _stream()))
+        int(bool(write_kv)), ctypes.c_float(unit_eps), _stream()))
 
 
 WINDOW_ATTENTION_MFMA = True     # steps with prompt portions take the matrix-instruction kernel (False: the FMA one, for comparison)
@@ -948,14 +954,22 @@ def window_attention_supported(H: int, Hkv: int, dk: int, dv: int) -> bool:
 def window_attention(q: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, dk: int, dv: int,
                      k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, page: int,
                      ctx, scale: float, window: int = 0, value_rotary=None,
-                     interleaved_values: bool = False, sink: Optional[torch.Tensor] = None) -> None:
+                     interleaved_values: bool = False, sink: Optional[torch.Tensor] = None,
+                     keep_first: int = 0, sigmoid_bias: Optional[torch.Tensor] = None) -> None:
     """Attention of the step's tokens (rotated queries ``q [T, H dk]``) over the cache into
     ``out [T, H dv]``: keys of size ``dk``, values of size ``dv``, the last ``window`` positions
     (0: all).  ``value_rotary``: the cached values are turned by their positions, and each sum is
     turned back by its query's.  ``sink`` (32-bit, one number a query head): ``exp(sink_h)`` joins the
-    softmax's denominator, with no key and no value."""
-    _dev(q, out, k_cache, v_cache, block_table, sink)
+    softmax's denominator, with no key and no value.  ``keep_first``: with a window, the first so many
+    positions of a request stay in sight of every later query.  ``sigmoid_bias`` (32-bit, one number a
+    query head): no softmax; a visible key's weight is ``sigmoid(score + sigmoid_bias[h])``, and the
+    weights are not normalised over the keys."""
+    _dev(q, out, k_cache, v_cache, block_table, sink, sigmoid_bias)
     _f32_vec(sink, H, "window_attention: the sink")
+    _f32_vec(sigmoid_bias, H, "window_attention: the sigmoids' bias")
+    if sink is not None and sigmoid_bias is not None:
+        raise KernelError("window_attention: sigmoid weights take no sink")
+    keep_first = int(keep_first) if window else 0
     _rows2d(q, "q")
     _rows2d(out, "out")
     T = q.shape[0]
@@ -975,20 +989,21 @@ def window_attention(q: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, dk: i
         _check(lib.ri_attention_window_mfma(
             _ptr(q), q.stride(0), _ptr(out), out.stride(0), _dt(q), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], page,
             H, Hkv, dk, dv, _ptr(block_table), block_table.shape[1], _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens),
-            ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)), _ptr(sink), _stream()))
+            ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)), _ptr(sink),
+            keep_first, _ptr(sigmoid_bias), _stream()))
         return
     # a step of single tokens divides each row's keys between blocks, through a workspace
     single, ws, need = int(ctx.max_q_len == 1 and T <= ctx.num_rows), None, 0
     if single:
         lib.ri_attention_window_workspace.restype = ctypes.c_size_t
-        need = lib.ri_attention_window_workspace(T, H, dk, dv, int(window), int(ctx.max_kv_len))
+        need = lib.ri_attention_window_workspace(T, H, dk, dv, int(window), int(ctx.max_kv_len), keep_first)
         if need:
             ws = ctx.workspace.get("attn.window_partials", need, 1, torch.float32)
     _check(lib.ri_attention_window(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _dt(q), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], page,
         H, Hkv, dk, dv, _ptr(block_table), block_table.shape[1], _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens),
         ctx.num_rows, T, ctypes.c_float(scale), int(window), vcos, vsin, vrows, int(bool(interleaved_values)),
-        single, int(ctx.max_kv_len), _ptr(ws), ctypes.c_size_t(need), _ptr(sink), _stream()))
+        single, int(ctx.max_kv_len), _ptr(ws), ctypes.c_size_t(need), _ptr(sink), keep_first, _ptr(sigmoid_bias), _stream()))
 
 
 # ---------------------------------------------------------------------------
@@ -1043,10 +1058,11 @@ def linear_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
 
 
 def gated_group_norm(o: torch.Tensor, weight: Optional[torch.Tensor], gate: Optional[torch.Tensor], out: torch.Tensor,
-                     group: int, eps: float, gate_activation: str = "sigmoid") -> None:
+                     group: int, eps: float, gate_activation: str = "sigmoid", gate_first: bool = False) -> None:
     """``out = o / sqrt(mean over each group of `group` features (o^2) + eps) * weight * sigmoid(gate)``;
     ``o`` 32-bit ``[T, n]``, ``gate`` and ``out`` activations (columns of wider buffers allowed).
-    ``weight = None``: no weight; ``gate_activation = "silu"``: ``silu(gate)`` in place of the sigmoid."""
+    ``weight = None``: no weight; ``gate_activation = "silu"``: ``silu(gate)`` in place of the sigmoid.
+    ``gate_first``: the gate multiplies ``o`` before the norm, ``out = norm(o * act(gate)) * weight``."""
     _dev(o, weight, gate, out)
     _rows2d(o, "o")
     _rows2d(out, "out")
@@ -1062,7 +1078,7 @@ def gated_group_norm(o: torch.Tensor, weight: Optional[torch.Tensor], gate: Opti
     _check(_lib().ri_gated_group_norm(_ptr(o), o.stride(0), T, n, int(group), _ptr(weight),
                                       _dt(weight) if weight is not None else F32, _ptr(gate),
                                       gate.stride(0) if gate is not None else 0, _ptr(out), out.stride(0), _dt(out),
-                                      ctypes.c_float(eps), int(gate_activation == "silu"), _stream()))
+                                      ctypes.c_float(eps), int(gate_activation == "silu"), int(bool(gate_first)), _stream()))
 
 
 # ---------------------------------------------------------------------------
@@ -1318,13 +1334,21 @@ SHORT_CONV_MAX_TAPS = 8
 SHORT_CONV_MAX_SEGMENTS = 4
 
 
-def short_conv(xs, ws, state: Optional[torch.Tensor], out: torch.Tensor, ctx, taps: int, silu: bool = True) -> None:
+def short_conv(xs, ws, state: Optional[torch.Tensor], out: torch.Tensor, ctx, taps: int, silu: bool = True,
+               biases=None) -> None:
     """A causal convolution over time of ``taps`` taps, channel by channel, through the last ``taps - 1``
     inputs each request keeps in ``state [slots, taps - 1, C]`` (32-bit; a request's first tokens start
     from zeros): ``xs`` are up to four ``[T, n_s]`` inputs (columns of a wider buffer allowed), ``ws`` their
     weights ``[n_s, taps]`` (the last column is the current token's); ``out [T, C]`` (32-bit, ``C`` the sum
-    of the ``n_s``) takes the results side by side, through silu if asked."""
+    of the ``n_s``) takes the results side by side, through silu if asked.  ``biases``: a 32-bit ``[n_s]``
+    (or None) for each input, added before the silu."""
     _dev(state, out, *xs, *ws)
+    if biases is not None:
+        if len(biases) != len(xs):
+            raise KernelError("short_conv: a bias (or None) for each input expected")
+        for b, x in zip(biases, xs):
+            _f32_vec(b, x.shape[1], "short_conv: a bias")
+        _dev(*[b for b in biases if b is not None])
     if not xs or len(xs) != len(ws) or len(xs) > SHORT_CONV_MAX_SEGMENTS:
         raise KernelError(f"short_conv: 1 to {SHORT_CONV_MAX_SEGMENTS} inputs with a weight each expected")
     _rows2d(out, "out")
@@ -1348,7 +1372,10 @@ def short_conv(xs, ws, state: Optional[torch.Tensor], out: torch.Tensor, ctx, ta
     wptrs = (ctypes.c_void_p * n)(*[w.data_ptr() for w in ws])
     strides = (ctypes.c_int * n)(*[x.stride(0) for x in xs])
     widths = (ctypes.c_int * n)(*[x.shape[1] for x in xs])
-    _check(_lib().ri_short_conv(n, ptrs, strides, wptrs, widths, _dt(xs[0]), int(taps), int(bool(silu)), _ptr(state),
+    bptrs = None
+    if biases is not None:
+        bptrs = (ctypes.c_void_p * n)(*[b.data_ptr() if b is not None else None for b in biases])
+    _check(_lib().ri_short_conv(n, ptrs, strides, wptrs, bptrs, widths, _dt(xs[0]), int(taps), int(bool(silu)), _ptr(state),
                                 state.shape[0] if state is not None else 1, _ptr(out), out.stride(0), _ptr(ctx.cu_q),
                                 _ptr(ctx.q_start), _ptr(ctx.state_slots), ctx.num_rows, T, int(ctx.max_q_len), _stream()))
 
@@ -1383,3 +1410,118 @@ def gated_delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta_in:
         _ptr(decay_in), decay_in.stride(0), _dt(beta_in), _ptr(A), _ptr(dt_bias), ctypes.c_float(unit_eps),
         ctypes.c_float(q_scale), _ptr(state), state.shape[0], _ptr(out), out.stride(0), _ptr(ctx.cu_q), _ptr(ctx.q_start),
         _ptr(ctx.state_slots), ctx.num_rows, T, H, Hk, dk, dv, _stream()))
+
+
+def _scan_common(state, out, ctx, H, dk, dv, T, who):
+    if tuple(out.shape) != (T, H * dv) or out.dtype != torch.float32:
+        raise KernelError(f"{who}: 32-bit out [T, {H * dv}] expected")
+    if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (H, dk, dv) or not state.is_contiguous():
+        raise KernelError(f"{who}: state must be contiguous float32 [slots, {H}, {dk}, {dv}]")
+    _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
+    _i32(ctx.q_start, "q_start", ctx.num_rows)
+    _i32(ctx.state_slots, "state_slots", ctx.num_rows)
+
+
+def channel_delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta_in: torch.Tensor, decay_in: torch.Tensor,
+                       A: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor, out: torch.Tensor, ctx,
+                       H: int, Hk: int, dk: int, dv: int, unit_eps: float = 1e-6, q_scale: float = 1.0) -> None:
+    """``gated_delta_scan`` with a decay for every key channel: ``S <- diag(g) S; u = beta (v - S^T k);
+    S <- S + k u^T; out = S^T q`` with ``g = exp(-A_h softplus(decay_in + dt_bias))`` laid out heads x dk
+    (``decay_in [T, H dk]`` activations, ``dt_bias [H dk]`` and ``A [H]`` 32-bit) and ``beta = sigmoid(beta_in)``,
+    ``beta_in [T, H]``.  q, k ``[T, Hk dk]`` and v ``[T, H dv]`` 32-bit; q and k are divided by
+    ``sqrt(|.|^2 + unit_eps)``, q also times ``q_scale``."""
+    _dev(q, k, v, beta_in, decay_in, A, dt_bias, state, out)
+    for t, name in ((q, "q"), (k, "k"), (v, "v"), (out, "out"), (beta_in, "beta_in"), (decay_in, "decay_in")):
+        _rows2d(t, name)
+    T = q.shape[0]
+    if tuple(q.shape) != (T, Hk * dk) or tuple(k.shape) != (T, Hk * dk) or tuple(v.shape) != (T, H * dv) \
+            or any(t.dtype != torch.float32 for t in (q, k, v)):
+        raise KernelError("channel_delta_scan: 32-bit q, k [T, Hk dk] and v [T, H dv] expected")
+    if tuple(beta_in.shape) != (T, H) or tuple(decay_in.shape) != (T, H * dk) or beta_in.dtype != decay_in.dtype:
+        raise KernelError("channel_delta_scan: beta_in [T, H] and decay_in [T, H dk] of one dtype expected")
+    _scan_common(state, out, ctx, H, dk, dv, T, "channel_delta_scan")
+    _f32_vec(A, H, "channel_delta_scan: A")
+    _f32_vec(dt_bias, H * dk, "channel_delta_scan: dt_bias")
+    _check(_lib().ri_channel_delta_scan(
+        _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(beta_in), beta_in.stride(0),
+        _ptr(decay_in), decay_in.stride(0), _dt(beta_in), _ptr(A), _ptr(dt_bias), ctypes.c_float(unit_eps),
+        ctypes.c_float(q_scale), _ptr(state), state.shape[0], _ptr(out), out.stride(0), _ptr(ctx.cu_q), _ptr(ctx.q_start),
+        _ptr(ctx.state_slots), ctx.num_rows, T, H, Hk, dk, dv, _stream()))
+
+
+def decay_scan(mode: str, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_in: torch.Tensor, bias: torch.Tensor,
+               state: torch.Tensor, out: torch.Tensor, ctx, H: int, Hk: int, dk: int, dv: int,
+               rate: Optional[torch.Tensor] = None, tau: float = 1.0, q_scale: float = 1.0,
+               skip: Optional[torch.Tensor] = None) -> None:
+    """Walk each request's tokens of the step through ``state[slot] [H, dk, dv]`` (32-bit):
+    ``S <- diag(w) S + k v^T``, ``out = S^T r (+ skip_h v)``, with a decay that depends on the token.
+    ``mode = "channel"``: ``w = sigmoid(decay_in + bias)^(1 / tau)`` for every key channel (``decay_in [T, H dk]``,
+    ``bias [H dk]``), r times ``q_scale``.  ``mode = "head"``: ``dt = softplus(decay_in + bias)`` (``decay_in [T, H]``,
+    ``bias [H]``), ``w = exp(-rate_h dt)`` for the whole head, k times dt; r, k ``[T, Hk dk]``, head h reading
+    head ``h // (H // Hk)``.  r, k, v of one dtype; ``decay_in`` an activation; ``bias, rate, skip`` 32-bit."""
+    if mode not in ("channel", "head"):
+        raise KernelError(f"decay_scan: unknown mode {mode!r}")
+    _dev(r, k, v, decay_in, bias, rate, skip, state, out)
+    for t, name in ((r, "r"), (k, "k"), (v, "v"), (out, "out"), (decay_in, "decay_in")):
+        _rows2d(t, name)
+    T = r.shape[0]
+    if tuple(r.shape) != (T, Hk * dk) or tuple(k.shape) != (T, Hk * dk) or tuple(v.shape) != (T, H * dv) \
+            or k.dtype != r.dtype or v.dtype != r.dtype:
+        raise KernelError("decay_scan: r, k [T, Hk dk] and v [T, H dv] of one dtype expected")
+    n_dec = H * dk if mode == "channel" else H
+    if tuple(decay_in.shape) != (T, n_dec):
+        raise KernelError(f"decay_scan: decay_in must be [T, {n_dec}]")
+    if mode == "channel" and Hk != H:
+        raise KernelError("decay_scan: a decay a key channel goes with a head of r and k for every head")
+    _scan_common(state, out, ctx, H, dk, dv, T, "decay_scan")
+    _f32_vec(bias, n_dec, "decay_scan: bias")
+    _f32_vec(skip, H, "decay_scan: skip")
+    if mode == "head":
+        if rate is None:
+            raise KernelError("decay_scan: a rate for each head expected")
+        _f32_vec(rate, H, "decay_scan: rate")
+    _check(_lib().ri_decay_scan(
+        1 if mode == "channel" else 2, _ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _dt(r),
+        _ptr(decay_in), decay_in.stride(0), _dt(decay_in), _ptr(bias), _ptr(rate), ctypes.c_float(1.0 / tau),
+        ctypes.c_float(q_scale), _ptr(skip), _ptr(state), state.shape[0], _ptr(out), out.stride(0), _ptr(ctx.cu_q),
+        _ptr(ctx.q_start), _ptr(ctx.state_slots), ctx.num_rows, T, H, Hk, dk, dv, _stream()))
+
+
+def token_shift(h: torch.Tensor, mix: torch.Tensor, state: torch.Tensor, out: torch.Tensor, ctx) -> None:
+    """``out[t] = h[t] + (h[t - 1] - h[t]) * mix`` with ``h[t - 1]`` the same request's previous token (zeros
+    before position 0); ``state [slots, d]`` (32-bit) keeps every request's last ``h`` from step to step.
+    ``h [T, d]`` contiguous 32-bit, ``mix [d]`` 32-bit, ``out [T, d]`` contiguous in the activations' dtype."""
+    _dev(h, mix, state, out)
+    T, d = h.shape
+    if h.dtype != torch.float32 or not h.is_contiguous() or tuple(out.shape) != (T, d) or not out.is_contiguous():
+        raise KernelError("token_shift: contiguous 32-bit h [T, d] and contiguous out [T, d] expected")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != d or not state.is_contiguous():
+        raise KernelError(f"token_shift: state must be contiguous float32 [slots, {d}]")
+    _f32_vec(mix, d, "token_shift: the mixing weights")
+    _i32(ctx.positions, "positions", T)
+    _i32(ctx.row_of_token, "row_of_token", T)
+    _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
+    _i32(ctx.state_slots, "state_slots", ctx.num_rows)
+    _check(_lib().ri_token_shift(_ptr(h), _ptr(mix), _ptr(state), state.shape[0], _ptr(out), _dt(out), T, d,
+                                 _ptr(ctx.positions), _ptr(ctx.row_of_token), _ptr(ctx.cu_q), _ptr(ctx.state_slots), _stream()))
+
+
+def stream_pair(x: torch.Tensor, delta: Optional[torch.Tensor], y: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[t] = [x[t] + delta[t] | y[t]]`` side by side, rounded to ``out``'s dtype: ``x [T, d]`` 32-bit,
+    ``delta`` ``[T, d]`` or a 32-bit stack ``[P, T, d]`` of partial sums (or None), ``y [T, d]`` 32-bit,
+    ``out [T, 2 d]``; all contiguous.  ``x`` itself is left as it is."""
+    _dev(x, delta, y, out)
+    T, d = x.shape
+    if x.dtype != torch.float32 or y.dtype != torch.float32 or tuple(y.shape) != (T, d) or tuple(out.shape) != (T, 2 * d) \
+            or not (x.is_contiguous() and y.is_contiguous() and out.is_contiguous()):
+        raise KernelError("stream_pair: contiguous 32-bit x, y [T, d] and contiguous out [T, 2 d] expected")
+    parts, stride, ddt = 1, 0, F32
+    if delta is not None:
+        if delta.dim() == 3:
+            parts, stride = delta.shape[0], delta.stride(0)
+        if delta.dim() not in (2, 3) or tuple(delta.shape[-2:]) != (T, d) or delta.stride(-1) != 1 or delta.stride(-2) != d \
+                or (delta.dim() == 3 and delta.dtype != torch.float32):
+            raise KernelError("stream_pair: delta must be [T, d] or a float32 stack [P, T, d] with contiguous rows")
+        ddt = _dt(delta)
+    _check(_lib().ri_stream_pair(_ptr(x), _ptr(delta), ddt, parts, ctypes.c_longlong(stride), _ptr(y), F32, _ptr(out),
+                                 _dt(out), T, d, _stream()))

@@ -121,9 +121,12 @@ class DecoderModel(Part):
         if self.keeps_embedded:
             # the rows as the embedding left them, for the parts that add them again later
             embedded = ws.get("model.embedded", T, self.hidden_size, torch.float32)
-            self.embed.forward(ctx, ctx.token_ids, embedded)
-            for pe in self.position_encodings:
-                pe.on_embedding(ctx, embedded)
+            if getattr(self.embed, "norm", None) is not None:
+                embedded.copy_(x)                # (the rows have passed a norm: a copy is cheaper than a second pass)
+            else:
+                self.embed.forward(ctx, ctx.token_ids, embedded)
+                for pe in self.position_encodings:
+                    pe.on_embedding(ctx, embedded)
         W = ctx.num_want
         # Only the rows whose logits are wanted matter after the last block's mixer: a long prompt
         # portion that wants one row (or none) runs that block's feed-forward on that row alone.
@@ -137,9 +140,14 @@ class DecoderModel(Part):
             cache = caches.view(call.cache, call.write) if call.cache in caches else None
             layer = self.layers[call.layer]
             if call.enter is not None:
-                if hidden.pending is not None or hidden.deferred is not None:
-                    raise RuntimeError("a part that acts on the stream between two layers needs the stream complete")
-                self.stream_parts[call.enter[0]][1].forward(ctx, hidden.x, embedded, call.enter[1])
+                part = self.stream_parts[call.enter[0]][1]
+                if getattr(part, "takes_hidden", False):
+                    # a part that deals with a pending sum itself (it reads the stream once and replaces it)
+                    part.forward(ctx, hidden, embedded, call.enter[1])
+                else:
+                    if hidden.pending is not None or hidden.deferred is not None:
+                        raise RuntimeError("a part that acts on the stream between two layers needs the stream complete")
+                    part.forward(ctx, hidden.x, embedded, call.enter[1])
                 hidden.act = None
             if n + 1 < len(self.schedule):
                 nxt = self.layers[self.schedule[n + 1].layer]

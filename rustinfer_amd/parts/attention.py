@@ -167,7 +167,16 @@ class WindowAttention(ProjectedPart, Mixer):
     ``<q>.norm``, ``<k>.norm``); the cache holds the normed keys.  ``q_temperature = (coef, every)``:
     the query at position p is multiplied by ``1 + coef ln(floor((p + 1) / every) + 1)``.  Either goes
     without a rotation of queries and keys.  ``own_kv = False``: the layer has no keys and values of
-    its own and reads a cache that another layer writes (the run order names it)."""
+    its own and reads a cache that another layer writes (the run order names it).
+
+    ``interleaved``: the checkpoint's rotation pairs feature 2i with 2i + 1; the rows of ``q`` and ``k`` that make
+    the turned features are reordered when they are loaded (even ones, then odd ones, head by head), which
+    leaves every score as it was.  ``qk_unit_eps``: after the rotation every head of q and k is divided by its
+    root mean square (this eps inside the root), with no weight.  ``keep_first``: behind the window the first so
+    many positions of a sequence stay in sight, at their true positions; the cache never gives their pages back.
+    ``sink``: a learned number a head (tensor ``sink``) whose exponential joins the softmax's denominator.
+    ``sigmoid_weights``: no softmax; a visible key's weight is ``sigmoid(score + b_h)`` with a learned number a
+    head (tensor ``pb``), and the weights are not normalised over the keys."""
 
     is_mixer = True
 
@@ -175,9 +184,20 @@ class WindowAttention(ProjectedPart, Mixer):
                  scale: float, window: Optional[int] = None, pos_enc: Optional[PositionEncoding] = None,
                  value_pos_enc: Optional[PositionEncoding] = None, interleaved_values: bool = False,
                  names: Optional[Dict[str, str]] = None, qk_norm_eps: Optional[float] = None,
-                 q_temperature=None, own_kv: bool = True):
+                 q_temperature=None, own_kv: bool = True, interleaved: bool = False,
+                 qk_unit_eps: Optional[float] = None, keep_first: int = 0, sink: bool = False,
+                 sigmoid_weights: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
+        if sink and sigmoid_weights:
+            raise ValueError("a sink belongs to a softmax: sigmoid weights take none")
+        if keep_first and not window:
+            keep_first = 0                       # without a window every position stays in sight anyway
+        self.interleaved = bool(interleaved)
+        self.qk_unit_eps = float(qk_unit_eps) if qk_unit_eps else None
+        self.keep_first = int(keep_first)
+        self.has_sink, self.sigmoid_weights = bool(sink), bool(sigmoid_weights)
+        self.sink = self.sigmoid_bias = None
         self.qk_norm_eps = float(qk_norm_eps) if qk_norm_eps is not None else None
         self.q_temperature = (float(q_temperature[0]), int(q_temperature[1])) if q_temperature else None
         self.own_kv = bool(own_kv)
@@ -191,9 +211,18 @@ class WindowAttention(ProjectedPart, Mixer):
         self.window = int(window) if window else None
         self.pos_enc, self.value_pos_enc = pos_enc, value_pos_enc
         self.interleaved_values = bool(interleaved_values)
-        self.names = {"q": "q", "k": "k", "v": "v", "o": "o"}
+        self.names = {"q": "q", "k": "k", "v": "v", "o": "o", "sink": "sink", "sigmoid_bias": "pb"}
         if names:
             self.names.update(names)
+        if self.by_head and (self.interleaved or self.qk_unit_eps is not None):
+            raise ValueError("the weighted norm of queries and keys goes without a rotation and without the unit norm")
+
+    def arrange_in(self, name: str, w: torch.Tensor) -> torch.Tensor:
+        rot = self.pos_enc.rot_dim if self.pos_enc is not None else 0
+        if not self.interleaved or rot == 0 or name not in (self.names["q"], self.names["k"]):
+            return w
+        heads = w.view(-1, self.head_dim, w.shape[1])
+        return torch.cat([heads[:, 0:rot:2], heads[:, 1:rot:2], heads[:, rot:]], dim=1).reshape(w.shape).contiguous()
 
     def in_projections(self):
         n = self.names
@@ -203,10 +232,14 @@ class WindowAttention(ProjectedPart, Mixer):
                 (n["v"], self.num_kv_heads * self.v_head_dim)]
 
     def own_specs(self):
+        n, specs = self.names, {}
+        if self.has_sink:
+            specs[n["sink"]] = ParamSpec((self.num_heads,), mean=0.0, std=1.0)
+        if self.sigmoid_weights:
+            specs[n["sigmoid_bias"]] = ParamSpec((self.num_heads,), mean=-2.0, std=1.0)
         if self.qk_norm_eps is None:
-            return {}
-        n = self.names
-        specs = {n["q"] + ".norm": ParamSpec((self.head_dim,), "norm")}
+            return specs
+        specs[n["q"] + ".norm"] = ParamSpec((self.head_dim,), "norm")
         if self.own_kv:
             specs[n["k"] + ".norm"] = ParamSpec((self.head_dim,), "norm")
         return specs
@@ -215,10 +248,15 @@ class WindowAttention(ProjectedPart, Mixer):
         return (self.names["o"], self.num_heads * self.v_head_dim)
 
     def cache_need(self):
-        return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window, self.v_head_dim)
+        return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window, self.v_head_dim, self.keep_first)
 
     def load_own(self, tensors, rt: Runtime) -> None:
         self.rt = rt
+        f32 = lambda name: tensors[name].to(device=rt.device, dtype=torch.float32).contiguous()
+        if self.has_sink:
+            self.sink = f32(self.names["sink"])
+        if self.sigmoid_weights:
+            self.sigmoid_bias = f32(self.names["sigmoid_bias"])
         if not rt.ops.window_attention_supported(self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim):
             raise ValueError(f"attention with {self.num_heads}/{self.num_kv_heads} heads of {self.head_dim} and "
                              f"{self.v_head_dim} features is beyond the window attention kernel")
@@ -244,11 +282,21 @@ class WindowAttention(ProjectedPart, Mixer):
             return
         rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
         vrot = self.value_pos_enc.rotary()[:2] if self.value_pos_enc is not None else None
+        extra = {}
+        if self.qk_unit_eps is not None:
+            extra["unit_eps"] = self.qk_unit_eps
         ops.rotate_kv_write(q, k, v, self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim, rotary, vrot,
                             ctx.positions, ctx.row_of_token, cache.k, cache.v, table, cache.page_size,
-                            write_kv=write, interleaved_values=self.interleaved_values)
+                            write_kv=write, interleaved_values=self.interleaved_values, **extra)
+        extra = {}
+        if self.sink is not None:
+            extra["sink"] = self.sink
+        if self.keep_first:
+            extra["keep_first"] = self.keep_first
+        if self.sigmoid_bias is not None:
+            extra["sigmoid_bias"] = self.sigmoid_bias
         ops.window_attention(q, act, self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim, cache.k, cache.v,
-                             table, cache.page_size, ctx, self.scale, self.window or 0, vrot, self.interleaved_values)
+                             table, cache.page_size, ctx, self.scale, self.window or 0, vrot, self.interleaved_values, **extra)
 
 
 class LatentAttention(ProjectedPart, Mixer):

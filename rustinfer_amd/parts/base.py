@@ -71,6 +71,7 @@ class PagedKVNeed:
     head_dim: int
     window: Optional[int] = None
     v_head_dim: Optional[int] = None
+    keep_first: int = 0       # with a window: the first so many positions stay readable, their pages are never given back
 
     @property
     def value_dim(self) -> int:
@@ -89,6 +90,35 @@ class StateNeed:
     def all_tensors(self):
         """[(name, shape, dtype)] of every tensor a slot holds; the main one is called ``""``."""
         return [("", tuple(self.shape), self.dtype)] + [(n, tuple(s), d) for n, s, d in self.extra]
+
+
+@dataclass(frozen=True)
+class CompoundNeed:
+    """What a layer asks for that keeps both a cache of keys and values and a fixed-size state (a mixer of
+    two halves, or an attention layer behind something that carries a row from token to token): the layer
+    gets a ``CompoundView`` with ``kv`` and ``state``."""
+    kv: PagedKVNeed
+    state: StateNeed
+
+
+def simple_needs(need):
+    """The ``PagedKVNeed`` / ``StateNeed`` a need is made of."""
+    if need is None:
+        return []
+    return [need.kv, need.state] if isinstance(need, CompoundNeed) else [need]
+
+
+def with_state_extra(need, name: str, shape, dtype=torch.float32):
+    """``need`` with one more tensor ``name`` in the request's state slot: a ``StateNeed`` gains an extra, a
+    ``PagedKVNeed`` becomes a ``CompoundNeed`` whose state has no main tensor of any size but this extra."""
+    extra = ((name, tuple(shape), dtype),)
+    if need is None:
+        return StateNeed((0,), torch.float32, extra)
+    if isinstance(need, StateNeed):
+        return StateNeed(need.shape, need.dtype, tuple(need.extra) + extra)
+    if isinstance(need, CompoundNeed):
+        return CompoundNeed(need.kv, with_state_extra(need.state, name, shape, dtype))
+    return CompoundNeed(need, StateNeed((0,), torch.float32, extra))
 
 
 @dataclass
@@ -344,12 +374,17 @@ class ProjectionSet:
     starts at a multiple of eight columns (16 bytes in bfloat16), the gaps being rows and columns
     of zeros."""
 
-    def __init__(self, hidden_size: int, members, extra_in=()):
+    def __init__(self, hidden_size: int, members, extra_in=(), out_scales=None):
         """``extra_in``: ``[(tensor name, rows)]`` of further projections of the same input that belong to
-        whoever owns the set (a gate on a sub-layer's result, say); their columns are ``extra_views``."""
+        whoever owns the set (a gate on a sub-layer's result, say); their columns are ``extra_views``.
+        ``out_scales``: a factor for each member's output (the sum is ``sum_i s_i W_out,i act_i``): the
+        member's columns of the stacked out-projection are multiplied by it, in 32-bit, when they are loaded."""
         from .linear import Linear
         self.hidden_size = int(hidden_size)
         self.members = list(members)                     # [(prefix, part)]
+        self.out_scales = [float(x) for x in out_scales] if out_scales is not None else None
+        if self.out_scales is not None and len(self.out_scales) != len(self.members):
+            raise ValueError("a factor for each member expected")
         self.in_slices, self.act_slices = [], []
         n_in = n_act = 0
         self.extra_slices = {}
@@ -390,11 +425,14 @@ class ProjectionSet:
             w_in[c0:c0 + rows] = tensors[name].to(device=rt.device, dtype=rt.dtype)
         w_out = torch.zeros((self.hidden_size, self.n_act), device=rt.device, dtype=rt.dtype)
         self._gaps, end = [], 0
-        for (prefix, part), views, (a0, cols) in zip(self.members, self.in_slices, self.act_slices):
+        for i, ((prefix, part), views, (a0, cols)) in enumerate(zip(self.members, self.in_slices, self.act_slices)):
             sub = narrow_tensors(tensors, prefix) if prefix else tensors
             for name, (c0, rows) in views.items():
                 w_in[c0:c0 + rows] = part.arrange_in(name, sub[name].to(device=rt.device, dtype=rt.dtype))
-            w_out[:, a0:a0 + cols] = sub[part.out_projection()[0]].to(device=rt.device, dtype=rt.dtype)
+            w_o = sub[part.out_projection()[0]].to(device=rt.device)
+            if self.out_scales is not None and self.out_scales[i] != 1.0:
+                w_o = w_o.to(torch.float32) * self.out_scales[i]
+            w_out[:, a0:a0 + cols] = w_o.to(rt.dtype)
             if a0 > end:
                 self._gaps.append((end, a0))
             end = a0 + cols

@@ -15,7 +15,8 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import FeedForward, Mixer, Norm, ParamSpec, Part, ProjectionSet, Runtime, join_name, narrow_tensors
+from .base import (FeedForward, Mixer, Norm, ParamSpec, Part, ProjectionSet, Runtime, join_name, narrow_tensors,
+                   with_state_extra)
 
 
 class Hidden:
@@ -44,23 +45,59 @@ class Hidden:
         return out
 
 
+class TokenShift(Part):
+    """What a sub-layer reads is mixed with what it read one token earlier, channel by channel:
+    ``h_t <- h_t + (h_(t-1) - h_t) * mix`` with ``h_(t-1)`` as it was before its own mixing, zeros before a
+    sequence's first token.  The last ``h`` of every request stays in its state slot (32-bit, the tensor
+    ``state_name`` there), so prompt portions and single tokens go the same way.  The tensor ``mix``
+    (the model's width) carries the part's own name."""
+
+    state_name = "shift"
+
+    def __init__(self, dim: int):
+        self.dim = int(dim)
+        self.mix = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {"": ParamSpec((self.dim,), mean=0.5, std=0.2)}
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.mix = tensors[""].to(device=rt.device, dtype=torch.float32).contiguous()
+
+    def state_of(self, cache):
+        state = getattr(cache, "state", None)
+        view = state if hasattr(state, "extra") else cache       # a CompoundView holds the StateView; a StateView is it
+        return view.extra[self.state_name]
+
+    def forward(self, ctx, h32: torch.Tensor, cache, out: torch.Tensor) -> torch.Tensor:
+        """``h32 [T, dim]``: the normed rows in 32-bit; ``out`` takes the mixed rows in the run dtype."""
+        self.rt.ops.token_shift(h32, self.mix, self.state_of(cache), out, ctx)
+        return out
+
+
 class PreNormBlock(Part):
     def __init__(self, hidden_size: int,
                  mixer_norm: Optional[Norm], mixer: Optional[Mixer],
                  ffn_norm: Optional[Norm], ffn: Optional[FeedForward],
-                 names: Optional[Dict[str, str]] = None):
+                 names: Optional[Dict[str, str]] = None, mixer_shift: Optional[TokenShift] = None):
+        """``mixer_shift``: a ``TokenShift`` between the mixer's norm and the mixer; the block then asks for
+        one more tensor in the request's state slot, beside whatever the mixer keeps."""
         self.hidden_size = int(hidden_size)
         self.mixer_norm, self.mixer = mixer_norm, mixer
         self.ffn_norm, self.ffn = ffn_norm, ffn
+        self.mixer_shift = mixer_shift
         if (mixer is None) != (mixer_norm is None) or (ffn is None) != (ffn_norm is None):
             raise ValueError("a sub-layer and its norm come together")
+        if mixer_shift is not None and mixer is None:
+            raise ValueError("a token shift stands in front of a mixer")
         self.names = {"mixer_norm": "input_layernorm", "mixer": "self_attn",
-                      "ffn_norm": "post_attention_layernorm", "ffn": "mlp"}
+                      "ffn_norm": "post_attention_layernorm", "ffn": "mlp", "mixer_shift": "shift"}
         if names:
             self.names.update(names)
 
     def _children(self):
-        for key in ("mixer_norm", "mixer", "ffn_norm", "ffn"):
+        for key in ("mixer_norm", "mixer_shift", "mixer", "ffn_norm", "ffn"):
             part = getattr(self, key)
             if part is not None:
                 yield self.names[key], part
@@ -79,7 +116,10 @@ class PreNormBlock(Part):
             part.load(sub, rt)
 
     def cache_need(self):
-        return self.mixer.cache_need() if self.mixer is not None else None
+        need = self.mixer.cache_need() if self.mixer is not None else None
+        if self.mixer_shift is not None:
+            need = with_state_extra(need, self.mixer_shift.state_name, (self.hidden_size,))
+        return need
 
     @property
     def graph_safe(self) -> bool:
@@ -93,7 +133,20 @@ class PreNormBlock(Part):
 
     def entry(self):
         """(norm, sub-layer) that a step enters this block through."""
+        if self.mixer_shift is not None:
+            return (self.mixer_norm, None)       # nobody else can prepare what the shift reads
         return (self.mixer_norm, self.mixer) if self.mixer is not None else (self.ffn_norm, self.ffn)
+
+    def _mixer_input(self, ctx, hidden: "Hidden", cache, normed: torch.Tensor):
+        """What the mixer reads: the normed rows, through the token shift if the block has one (the norm then
+        leaves 32-bit rows, and the shift rounds once)."""
+        if self.mixer_shift is None:
+            return hidden.input_behind(ctx, self.mixer_norm, normed)
+        h32 = ctx.workspace.get("block.normed32", normed.shape[0], self.hidden_size, torch.float32)
+        hidden.deferred = None
+        self.mixer_norm.forward(ctx, hidden.x, hidden.pending, h32)
+        hidden.pending = None
+        return self.mixer_shift.forward(ctx, h32, cache, normed)
 
     def forward(self, ctx, hidden: Hidden, cache, out_rows: Optional[torch.Tensor] = None, follow=None) -> None:
         """``out_rows`` (row indices on the device): nothing after this block needs the other
@@ -105,7 +158,7 @@ class PreNormBlock(Part):
         T = hidden.x.shape[0]
         normed = ctx.workspace.get("block.normed", T, self.hidden_size, self.rt.dtype)
         if self.mixer is not None:
-            inp = hidden.input_behind(ctx, self.mixer_norm, normed)
+            inp = self._mixer_input(ctx, hidden, cache, normed)
             after = (self.ffn_norm, self.ffn) if self.ffn is not None else follow
             self._run(self.mixer, ctx, hidden, inp, after if out_rows is None or self.ffn is None else None, cache)
         if self.ffn is not None:
@@ -128,7 +181,7 @@ class PreNormBlock(Part):
         if self.mixer is None:
             return
         normed = ctx.workspace.get("block.normed", hidden.x.shape[0], self.hidden_size, self.rt.dtype)
-        inp = hidden.input_behind(ctx, self.mixer_norm, normed)
+        inp = self._mixer_input(ctx, hidden, cache, normed)
         update = getattr(self.mixer, "update_cache", None)
         if update is not None:
             update(ctx, inp, cache)
@@ -417,3 +470,46 @@ class SandwichBlock(Part):
         """The last block of a step whose logits nobody wants: the mixer alone runs, for what it leaves in
         its cache or state; ``hidden`` is not meaningful afterwards."""
         self._run_half(ctx, hidden, self.halves[0], cache, None, only_state=True)
+
+
+class TwoMixers(Mixer):
+    """A mixer made of two that read the same rows side by side: ``left_scale * left(h) + right_scale * right(h)``.
+    Both halves are ``ProjectedPart``: their input projections are one product, their output projections one
+    product over the activations side by side, with each half's factor in its columns of that weight.  The left
+    half keeps keys and values in pages, the right half a state of fixed size: the mixer asks for both
+    (``CompoundNeed``) and hands each half its own.  Tensors: the halves' under ``left.`` and ``right.``."""
+
+    def __init__(self, hidden_size: int, left, right, left_scale: float = 1.0, right_scale: float = 1.0,
+                 names: Optional[Dict[str, str]] = None):
+        from .base import CompoundNeed, PagedKVNeed, StateNeed
+        self.hidden_size = int(hidden_size)
+        self.left, self.right = left, right
+        self.names = {"left": "left", "right": "right"}
+        if names:
+            self.names.update(names)
+        self.set = ProjectionSet(self.hidden_size, [(self.names["left"], left), (self.names["right"], right)],
+                                 out_scales=[left_scale, right_scale])
+        kv, state = left.cache_need(), right.cache_need()
+        if not isinstance(kv, PagedKVNeed) or not isinstance(state, StateNeed):
+            raise ValueError("the left half keeps pages of keys and values, the right half a state of fixed size")
+        self._need = CompoundNeed(kv, state)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return self.set.param_specs()
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.set.load(tensors, rt)
+
+    def cache_need(self):
+        return self._need
+
+    @property
+    def graph_safe(self) -> bool:
+        return getattr(self.left, "graph_safe", True) and getattr(self.right, "graph_safe", True)
+
+    def forward(self, ctx, normed, cache) -> torch.Tensor:
+        proj, act = self.set.project(ctx, normed)
+        self.left.core(ctx, self.set.views(0, proj), self.set.act_view(0, act), cache.kv)
+        self.right.core(ctx, self.set.views(1, proj), self.set.act_view(1, act), cache.state)
+        return self.set.output(ctx, act)

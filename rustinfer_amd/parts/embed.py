@@ -15,25 +15,36 @@ from .base import ParamSpec, Part, Runtime, split_normed, stored_to
 
 
 class Embedding(Part):
-    def __init__(self, vocab_size: int, dim: int, weight_name: str = "weight", scale: float = 1.0):
+    def __init__(self, vocab_size: int, dim: int, weight_name: str = "weight", scale: float = 1.0, norm=None):
         self.vocab_size = int(vocab_size)
         self.dim = int(dim)
         self.weight = None
         self.weight_name = weight_name       # "" where the table carries the part's own name
         self.scale = float(scale)            # every embedded row is multiplied by it
+        self.norm = norm                     # a norm the embedded rows pass (its tensors under the table's name)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {self.weight_name: ParamSpec((self.vocab_size, self.dim), "matrix")}
+        specs = {self.weight_name: ParamSpec((self.vocab_size, self.dim), "matrix")}
+        if self.norm is not None:
+            specs.update(self.norm.param_specs())
+        return specs
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         self.weight = stored_to(tensors[self.weight_name], rt)
+        if self.norm is not None:
+            self.norm.load(tensors, rt)
 
     def forward(self, ctx, ids: torch.Tensor, out_x: torch.Tensor) -> torch.Tensor:
+        rows = out_x
+        if self.norm is not None:
+            rows = ctx.workspace.get("embed.rows", out_x.shape[0], self.dim, torch.float32)
         if self.scale != 1.0:
-            self.rt.ops.embed(ids, self.weight, out_x, getattr(ctx, "device_tokens", None), scale=self.scale)
+            self.rt.ops.embed(ids, self.weight, rows, getattr(ctx, "device_tokens", None), scale=self.scale)
         else:
-            self.rt.ops.embed(ids, self.weight, out_x, getattr(ctx, "device_tokens", None))
+            self.rt.ops.embed(ids, self.weight, rows, getattr(ctx, "device_tokens", None))
+        if self.norm is not None:
+            self.norm.forward(ctx, rows, None, out_x)          # 32-bit rows in, 32-bit stream out
         return out_x
 
 

@@ -17,15 +17,25 @@ from .base import Norm, ParamSpec, Runtime, stored_to
 
 
 class RMSNorm(Norm):
-    def __init__(self, dim: int, eps: float, weight_name: str = "weight", one_plus: bool = False):
+    def __init__(self, dim: int, eps: float, weight_name: str = "weight", one_plus: bool = False, groups: int = 1,
+                 weight_32bit: bool = False):
         """``weight_name``: the weight's name under the norm's own ("" where the tensor carries the
         norm's name itself).  ``one_plus``: the checkpoint stores the weight around zero and the norm
-        multiplies by ``1 + w`` (kept as that sum, in 32-bit)."""
+        multiplies by ``1 + w`` (kept as that sum, in 32-bit).  ``groups``: a row is split into that many
+        equal consecutive parts and each is divided by its own root mean square.  ``weight_32bit``: the weight is
+        widened to 32-bit whatever the checkpoint stores (for norms whose rows leave in 32-bit)."""
+        self.weight_32bit = bool(weight_32bit)
         self.dim = int(dim)
         self.eps = float(eps)
         self.weight = None
         self.weight_name = weight_name
         self.one_plus = bool(one_plus)
+        self.groups = int(groups)
+        if self.groups < 1 or self.dim % self.groups:
+            raise ValueError(f"{self.dim} values do not split into {self.groups} equal parts")
+        # nothing but ``weight`` and ``eps``: the sub-layers around this norm may do it between them
+        # (``forward_into`` and ``DeferredNorm``, see PreNormBlock.forward); not so a norm in parts
+        self.plain_rms = self.groups == 1
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         if self.one_plus:
@@ -36,16 +46,18 @@ class RMSNorm(Norm):
         self.rt = rt
         if self.one_plus:
             self.weight = (tensors[self.weight_name].to(device=rt.device, dtype=torch.float32) + 1.0).contiguous()
+        elif self.weight_32bit:
+            self.weight = tensors[self.weight_name].to(device=rt.device, dtype=torch.float32).contiguous()
         else:
             self.weight = stored_to(tensors[self.weight_name], rt, keep_fp32=True)
 
     cuts_rows = True          # forward() takes x_rows (see PreNormBlock.forward)
-    # nothing but ``weight`` and ``eps``: the sub-layers around this norm may do it between them
-    # (``forward_into`` and ``DeferredNorm``, see PreNormBlock.forward)
-    plain_rms = True
 
     def forward(self, ctx, x, delta, out, rows=None, x_rows=None):
-        self.rt.ops.add_rmsnorm(x, delta, self.weight, self.eps, out, rows, x_rows)
+        if self.groups > 1:
+            self.rt.ops.add_rmsnorm(x, delta, self.weight, self.eps, out, rows, x_rows, groups=self.groups)
+        else:
+            self.rt.ops.add_rmsnorm(x, delta, self.weight, self.eps, out, rows, x_rows)
         return out
 
 
