@@ -479,6 +479,8 @@ class TwoMixers(Mixer):
     half keeps keys and values in pages, the right half a state of fixed size: the mixer asks for both
     (``CompoundNeed``) and hands each half its own.  Tensors: the halves' under ``left.`` and ``right.``."""
 
+    is_mixer = True
+
     def __init__(self, hidden_size: int, left, right, left_scale: float = 1.0, right_scale: float = 1.0,
                  names: Optional[Dict[str, str]] = None):
         from .base import CompoundNeed, PagedKVNeed, StateNeed

@@ -1,0 +1,640 @@
+"""Debuzen on the GPU against the plain implementation (``plain_debuzen.py``): every mechanism alone, then
+whole models of three small configurations that differ in every size, in the order of their layers, in the
+norm's groups and in the stretch that runs again, through every way of cutting requests into steps, through
+pages and state slots that are used again, and through ``LLM.generate``.  Weights are drawn here with
+deviations that make activations of order one; a few tests build inputs so that one key at a window's edge
+or among the kept first positions decides."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_debuzen as P
+from helpers import cut_mixed, cut_portions, cut_tail_single, cut_whole, random_requests, run_steps
+from test_gpu_belorax import CUTS, PART_TOL, Rows, check_rows, portion_kernel, rel, run_part, some_rows  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def att(heads, kv, dim, vdim, scale, size, dims, base=10000.0, keep=None):
+    mask = dict(size=size)
+    if keep is not None:
+        mask["keep_first"] = keep
+    return dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=scale, mask=mask, rot=dict(base=base, dims=dims))
+
+
+def par(left, heads, kv, dim, vdim, conv, ls=1.0, rs=1.0):
+    return dict(type="parallel", mixer=dict(left=left, right=dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, conv=conv),
+                                            left_scale=ls, right_scale=rs))
+
+
+def par2(left, heads, vdim, state, groups, conv, norm_groups, ls=1.0, rs=1.0):
+    return dict(type="parallel_2", mixer=dict(left=left, right=dict(heads=heads, vdim=vdim, state=state, groups=groups, conv=conv,
+                                                                    norm_groups=norm_groups), left_scale=ls, right_scale=rs))
+
+
+def gla(heads, dim, vdim, tau):
+    return dict(type="gla", mixer=dict(heads=heads, dim=dim, vdim=vdim, tau=tau))
+
+
+def layer(mixer, ff):
+    return dict(mixer, mlp=None if ff is None else dict(kind="dense", ff=ff))
+
+
+CONFIGS = {
+    # the stretch is the first two layers, three times; windows of a page and a bit; kept positions within one page; a layer without feed-forward
+    "A": dict(architecture="Debuzen", vocab=200, width=64, norm=dict(eps=1e-5, groups=4), logit_softcap=8.0,
+              loop=dict(start=0, stop=2, times=3), layers=[
+        layer(par(att(4, 2, 12, 8, 0.3, 11, 4, base=50.0, keep=3), 4, 2, 16, 8, 2, ls=0.7, rs=1.3), 96),
+        layer(gla(3, 8, 12, 4.0), None),
+        layer(par2(att(3, 1, 16, 10, 0.25, 19, 16, base=1000.0), 4, 8, 12, 2, 3, 2, ls=1.1, rs=0.4), 40),
+        layer(gla(2, 24, 40, 16.0), 50),
+    ]),
+    # no stretch; heads beyond one 64-wide slice, kept positions beyond a block of keys, a norm over whole rows, no soft cap
+    "B": dict(architecture="Debuzen", vocab=333, width=136, norm=dict(eps=1e-6, groups=1), logit_softcap=0.0, layers=[
+        layer(par2(att(6, 6, 40, 72, 0.1, 64, 12, base=200.0), 6, 40, 72, 1, 4, 1, ls=0.5, rs=0.5), 200),
+        layer(par(att(5, 1, 72, 132, 0.08, 33, 72, base=5e5, keep=70), 6, 1, 72, 36, 3, ls=1.0, rs=2.0), 64),
+        layer(gla(1, 130, 20, 2.0), None),
+        layer(par(att(2, 2, 24, 24, 0.2, 100, 8, keep=0), 3, 3, 128, 40, 1, ls=1.5, rs=0.25), 80),
+        layer(par2(att(8, 2, 16, 16, 0.25, 200, 16), 5, 24, 130, 5, 8, 3, ls=1.0, rs=1.0), None),
+    ]),
+    # a width and a vocabulary that are no multiples of eight; the stretch is one layer in the middle, twice; a window of one
+    "C": dict(architecture="Debuzen", vocab=211, width=100, norm=dict(eps=1e-6, groups=5), logit_softcap=30.0,
+              loop=dict(start=2, stop=3, times=2), layers=[
+        layer(gla(5, 20, 12, 1.0), 50),
+        layer(par2(att(1, 1, 12, 10, 0.4, 1, 2, base=20.0), 12, 6, 16, 4, 2, 6, ls=0.9, rs=0.9), 77),
+        layer(par(att(6, 3, 10, 14, 0.3, 40, 10, base=500.0, keep=17), 12, 2, 16, 18, 5, ls=0.6, rs=0.5), 33),
+        layer(par2(att(4, 4, 20, 6, 0.2, 16, 4), 2, 50, 20, 2, 1, 4, ls=1.2, rs=0.7), 64),
+    ]),
+}
+PAGE = {"A": 8, "B": 16, "C": 16}
+DECAY_RANK, GATE_RANK = 5, 7       # inner sizes of the pairs of matrices: the engine reads them from the shapes
+
+
+def bf16(a) -> torch.Tensor:
+    return torch.as_tensor(np.asarray(a), dtype=torch.float32).to(torch.bfloat16)
+
+
+def draw_attention(rng, m, W, p, t, sigmoid):
+    mat = lambda o, i, s=1.0: bf16(s * rng.standard_normal((o, i)) / math.sqrt(i))
+    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    t[p + "q"], t[p + "k"], t[p + "v"], t[p + "o"] = mat(H * d, W, 2.0), mat(G * d, W, 2.0), mat(G * dv, W), mat(W, H * dv)
+    if sigmoid:
+        t[p + "pb"] = bf16(-1.0 + rng.standard_normal(H))
+    else:
+        t[p + "sink"] = bf16(1.0 + 1.5 * rng.standard_normal(H))
+
+
+def draw_mixer(rng, m, kind, W, p, t):
+    mat = lambda o, i, s=1.0: bf16(s * rng.standard_normal((o, i)) / math.sqrt(i))
+    vec = lambda n, mean, std: bf16(mean + std * rng.standard_normal(n))
+    if kind == "gla":
+        H, d, dv = m["heads"], m["dim"], m["vdim"]
+        t[p + "q"], t[p + "k"], t[p + "v"], t[p + "g"] = mat(H * d, W, 2.0), mat(H * d, W), mat(H * dv, W), mat(H * dv, W)
+        t[p + "a1"], t[p + "a2"], t[p + "a2.b"] = mat(DECAY_RANK, W), mat(H * d, DECAY_RANK, 2.0), vec(H * d, 2.0, 1.0)
+        t[p + "o"], t[p + "norm"] = mat(W, H * dv), vec(dv, 1.0, 0.2)
+        return
+    draw_attention(rng, m["left"], W, p + "left.", t, kind == "parallel")
+    r, p = m["right"], p + "right."
+    if kind == "parallel":
+        H, Hk, dk, dv, taps = r["heads"], r["kv_heads"], r["dim"], r["vdim"], r["conv"]
+        for x, rows in (("q", Hk * dk), ("k", Hk * dk), ("v", H * dv)):
+            t[p + x], t[p + x + ".conv"] = mat(rows, W, 2.0), bf16(rng.standard_normal((rows, taps)) * 0.6)
+        t[p + "b"], t[p + "o"] = mat(H, W, 2.0), mat(W, H * dv)
+        t[p + "a1"], t[p + "a2"], t[p + "dt_bias"] = mat(DECAY_RANK, W), mat(H * dk, DECAY_RANK, 2.0), vec(H * dk, 0.0, 1.0)
+        t[p + "g1"], t[p + "g2"] = mat(GATE_RANK, W), mat(H * dv, GATE_RANK, 2.0)
+        t[p + "A_log"], t[p + "norm"] = vec(H, -1.0, 1.0), vec(dv, 1.0, 0.2)
+    else:
+        H, dv, N, G, taps = r["heads"], r["vdim"], r["state"], r["groups"], r["conv"]
+        inner, C = H * dv, H * dv + 2 * G * N
+        t[p + "in"] = mat(2 * inner + 2 * G * N + H, W, 1.5)
+        t[p + "conv"], t[p + "conv.b"] = bf16(rng.standard_normal((C, taps)) * 0.6), vec(C, 0.0, 0.3)
+        t[p + "dt_bias"], t[p + "A_log"], t[p + "D"] = vec(H, 0.0, 1.0), vec(H, -1.0, 1.0), vec(H, 1.0, 0.5)
+        t[p + "norm"], t[p + "o"] = vec(inner, 1.0, 0.2), mat(W, inner)
+
+
+def draw_weights(cfg: dict, seed: int):
+    """name -> bfloat16 tensor for every tensor of the design, activations of order one."""
+    rng = np.random.default_rng(seed)
+    W = cfg["width"]
+    mat = lambda o, i, s=1.0: bf16(s * rng.standard_normal((o, i)) / math.sqrt(i))
+    vec = lambda n, mean, std: bf16(mean + std * rng.standard_normal(n))
+    t = {"embed": bf16(rng.standard_normal((cfg["vocab"], W))), "embed.norm": vec(W, 1.0, 0.1), "final.norm": vec(W, 1.0, 0.1),
+         "head": mat(cfg["vocab"], W)}
+    if "loop" in cfg:
+        t["loop.in"] = mat(W, 2 * W, 1.4)
+    for i, lay in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        t[p + "norm1"], t[p + "shift"] = vec(W, 1.0, 0.1), bf16(rng.uniform(0.0, 1.0, W))
+        draw_mixer(rng, lay["mixer"], lay["type"], W, p + "mix.", t)
+        if lay["mlp"] is not None:
+            ff = lay["mlp"]["ff"]
+            t[p + "norm2"] = vec(W, 1.0, 0.1)
+            t[p + "mlp.gate"], t[p + "mlp.up"], t[p + "mlp.down"] = mat(ff, W), mat(ff, W), mat(W, ff)
+    return t
+
+
+@pytest.fixture(scope="module")
+def tdirs(tmp_path_factory):
+    from rustinfer_amd.weights import write_safetensors
+    out = {}
+    for k, (name, cfg) in enumerate(CONFIGS.items()):
+        d = str(tmp_path_factory.mktemp("debuzen_" + name))
+        with open(os.path.join(d, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        write_safetensors(os.path.join(d, "model.safetensors"), draw_weights(cfg, 81 + k))
+        out[name] = d
+    return out
+
+
+@pytest.fixture(scope="module")
+def plain(tdirs):
+    from safetensors.torch import load_file
+    return {name: (CONFIGS[name], load_file(os.path.join(d, "model.safetensors"))) for name, d in tdirs.items()}
+
+
+def plain_rows(cfg, w, reqs):
+    return Rows({rid: P.forward(cfg, w, toks).numpy() for rid, toks in reqs.items()})
+
+
+@pytest.fixture(scope="module")
+def plain_logits(plain):
+    memo = {}
+
+    def get(name, lengths, seed):
+        key = (name, tuple(lengths), seed)
+        if key not in memo:
+            cfg, w = plain[name]
+            reqs = random_requests(cfg["vocab"], lengths, seed)
+            memo[key] = (reqs, plain_rows(cfg, w, reqs))
+        return memo[key]
+    return get
+
+
+def engine_for(model_dir, dtype, name, num_pages=64, max_requests=4, max_len=512):
+    from rustinfer_amd.engine import build_engine
+    return build_engine(model_dir, dtype=dtype, device=DEV, page_size=PAGE[name], num_pages=num_pages,
+                        max_requests=max_requests, max_model_len=max_len, max_batch_tokens=2048)
+
+
+# ---------------------------------------------------------------------------
+# each mechanism alone
+# ---------------------------------------------------------------------------
+def load_part(part, wt, dtype):
+    from rustinfer_amd.engine import make_runtime
+    assert set(wt) == set(part.param_specs())
+    part.load(wt, make_runtime(dtype, DEV))
+    return {n: t.double() for n, t in wt.items()}
+
+
+def attention_part(width, m, sigmoid, eps=1e-5):
+    from rustinfer_amd.parts import RotaryEmbedding, WindowAttention
+    pe = RotaryEmbedding(m["dim"], m["rot"]["base"], rot_dim=m["rot"]["dims"])
+    part = WindowAttention(width, m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"], window=m["mask"]["size"], pos_enc=pe,
+                           interleaved=sigmoid, qk_unit_eps=eps if sigmoid else None, keep_first=m["mask"].get("keep_first", 0) if sigmoid else 0,
+                           sink=not sigmoid, sigmoid_weights=sigmoid)
+    return part, pe
+
+
+ATT_SIZES = [(4, 2, 12, 8, 11, 4, 3), (5, 1, 72, 132, 33, 72, 70), (2, 2, 24, 24, 100, 8, 0), (6, 3, 10, 14, 40, 10, 17), (1, 1, 12, 10, 1, 2, 2),
+             (8, 2, 64, 64, 64, 32, 64), (16, 1, 32, 16, 17, 16, 130), (3, 3, 80, 48, 128, 40, 9)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,dk,dv,size,dims,keep", ATT_SIZES)
+def test_attention_with_sigmoid_weights_and_kept_first_positions_alone(dtype, H, G, dk, dv, size, dims, keep, portion_kernel):
+    width = 56
+    m = att(H, G, dk, dv, 2.0 / math.sqrt(dk), size, dims, base=300.0, keep=keep)
+    part, pe = attention_part(width, m, True)
+    t = {}
+    draw_attention(np.random.default_rng(H * dk + size), m, width, "", t, True)
+    w = load_part(part, t, dtype)
+    x = some_rows(sum(CUTS), width, 6)
+    ref = P.sigmoid_attention(x.double(), w, m, 1e-5).numpy()
+    if 0 < keep and size + keep < sum(CUTS):
+        assert rel(P.sigmoid_attention(x.double(), w, dict(m, mask=dict(size=size)), 1e-5).numpy(), ref) > 0.02    # the kept positions matter
+    assert rel(run_part(part, [pe], dtype, x, CUTS), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [pe], dtype, x, [sum(CUTS)], page=16), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [pe], dtype, x, CUTS, batch_with=some_rows(60, width, 8)), ref) < PART_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,dk,dv,size,dims,keep", ATT_SIZES)
+def test_attention_with_a_sink_alone(dtype, H, G, dk, dv, size, dims, keep, portion_kernel):
+    width = 56
+    m = att(H, G, dk, dv, 2.0 / math.sqrt(dk), size, dims, base=300.0)
+    part, pe = attention_part(width, m, False)
+    t = {}
+    draw_attention(np.random.default_rng(H * dk + size), m, width, "", t, False)
+    w = load_part(part, t, dtype)
+    x = some_rows(sum(CUTS), width, 6)
+    ref = P.sink_attention(x.double(), w, m).numpy()
+    assert rel(P.sink_attention(x.double(), dict(w, sink=torch.full((H,), -1e9, dtype=torch.float64)), m).numpy(), ref) > 0.02
+    assert rel(run_part(part, [pe], dtype, x, CUTS), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [pe], dtype, x, [sum(CUTS)], page=16), ref) < PART_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,Hk,dk,dv,taps", [(4, 2, 16, 8, 2), (6, 1, 72, 36, 3), (3, 3, 128, 40, 1), (1, 1, 130, 20, 8),
+                                             (12, 2, 16, 18, 5), (2, 2, 256, 64, 4), (4, 4, 48, 80, 3)])
+def test_channel_gated_delta_rule_alone(dtype, H, Hk, dk, dv, taps):
+    from rustinfer_amd.parts import ChannelGatedDeltaRule
+    width = 40
+    r = dict(heads=H, kv_heads=Hk, dim=dk, vdim=dv, conv=taps)
+    part = ChannelGatedDeltaRule(width, H, Hk, dk, dv, taps, DECAY_RANK, GATE_RANK, 1e-5)
+    t = {}
+    draw_mixer(np.random.default_rng(H * dk + dv), dict(left=att(1, 1, 8, 8, 1.0, 4, 2), right=r), "parallel", width, "", t)
+    w = load_part(part, {n[6:]: v for n, v in t.items() if n.startswith("right.")}, dtype)
+    x = some_rows(sum(CUTS), width, 7)
+    ref = P.gated_delta(x.double(), w, r, 1e-5).numpy()
+    assert rel(run_part(part, [], dtype, x, CUTS), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [], dtype, x, CUTS, batch_with=some_rows(60, width, 8)), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [], dtype, x, [sum(CUTS)]), ref) < PART_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,dv,N,G,taps,ng", [(4, 8, 12, 2, 3, 2), (6, 40, 72, 1, 4, 1), (5, 24, 130, 5, 8, 3), (12, 6, 16, 4, 2, 6),
+                                              (2, 50, 20, 2, 1, 4), (6, 16, 40, 3, 4, 2), (3, 200, 256, 3, 4, 1)])
+def test_state_space_mixer_alone(dtype, H, dv, N, G, taps, ng):
+    from rustinfer_amd.parts import StateSpaceMixer
+    width = 40
+    r = dict(heads=H, vdim=dv, state=N, groups=G, conv=taps, norm_groups=ng)
+    part = StateSpaceMixer(width, H, dv, N, G, taps, ng, 1e-5)
+    t = {}
+    draw_mixer(np.random.default_rng(H * dv + N), dict(left=att(1, 1, 8, 8, 1.0, 4, 2), right=r), "parallel_2", width, "", t)
+    w = load_part(part, {n[6:]: v for n, v in t.items() if n.startswith("right.")}, dtype)
+    x = some_rows(sum(CUTS), width, 7)
+    ref = P.state_space(x.double(), w, r, 1e-5).numpy()
+    assert rel(run_part(part, [], dtype, x, CUTS), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [], dtype, x, CUTS, batch_with=some_rows(60, width, 8)), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [], dtype, x, [sum(CUTS)]), ref) < PART_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,dk,dv,tau", [(3, 8, 12, 4.0), (2, 24, 40, 16.0), (1, 130, 20, 2.0), (5, 20, 12, 1.0), (6, 40, 48, 16.0), (2, 256, 130, 8.0)])
+def test_gated_linear_attention_alone(dtype, H, dk, dv, tau):
+    from rustinfer_amd.parts import GatedLinearAttention
+    width = 40
+    m = dict(heads=H, dim=dk, vdim=dv, tau=tau)
+    part = GatedLinearAttention(width, H, dk, dv, tau, DECAY_RANK, 1e-5)
+    t = {}
+    draw_mixer(np.random.default_rng(H * dk + dv), m, "gla", width, "", t)
+    w = load_part(part, t, dtype)
+    x = some_rows(sum(CUTS), width, 7)
+    ref = P.gated_linear_attention(x.double(), w, m, 1e-5).numpy()
+    assert rel(run_part(part, [], dtype, x, CUTS), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [], dtype, x, CUTS, batch_with=some_rows(60, width, 8)), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [], dtype, x, [sum(CUTS)]), ref) < PART_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind", ["parallel", "parallel_2"])
+def test_two_mixers_side_by_side(dtype, kind, portion_kernel):
+    from rustinfer_amd.parts import ChannelGatedDeltaRule, StateSpaceMixer, TwoMixers
+    width = 48
+    left = att(4, 2, 16, 12, 0.4, 21, 8, base=100.0, keep=5 if kind == "parallel" else None)
+    if kind == "parallel":
+        right = dict(heads=3, kv_heads=1, dim=24, vdim=20, conv=3)
+        rpart = ChannelGatedDeltaRule(width, 3, 1, 24, 20, 3, DECAY_RANK, GATE_RANK, 1e-5)
+    else:
+        right = dict(heads=4, vdim=12, state=20, groups=2, conv=4, norm_groups=3)
+        rpart = StateSpaceMixer(width, 4, 12, 20, 2, 4, 3, 1e-5)
+    m = dict(left=left, right=right, left_scale=0.6, right_scale=1.7)
+    lpart, pe = attention_part(width, left, kind == "parallel")
+    part = TwoMixers(width, lpart, rpart, 0.6, 1.7)
+    t = {}
+    draw_mixer(np.random.default_rng(3), m, kind, width, "", t)
+    w = load_part(part, t, dtype)
+    x = some_rows(sum(CUTS), width, 5)
+    ref = P.mixer(kind, x.double(), w, m, 1e-5).numpy()
+    assert rel(P.mixer(kind, x.double(), w, dict(m, left_scale=1.0), 1e-5).numpy(), ref) > 0.02      # the factors matter
+    assert rel(run_part(part, [pe], dtype, x, CUTS), ref) < PART_TOL[dtype]
+    assert rel(run_part(part, [pe], dtype, x, [sum(CUTS)], page=16), ref) < PART_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width,groups,parts,T", [(64, 4, 1, 9), (100, 5, 3, 9), (4096, 2, 2, 9), (33, 3, 1, 9), (1024, 1, 8, 3),
+                                                  (192, 2, 1, 300), (1536, 6, 2, 260), (18, 9, 1, 5)])
+def test_the_norm_in_groups(dtype, width, groups, parts, T):
+    """Parts that do and do not allow loads of four values, partial sums, rows picked out, 32-bit and rounded results."""
+    from rustinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(width + groups)
+    act = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    x = torch.randn(T, width, generator=g) * 3.0 + 1.0
+    w = (1.0 + 0.3 * torch.randn(width, generator=g)).to(DEV)
+    delta = torch.randn(parts, T, width, generator=g)
+    d_in = delta if parts > 1 else delta[0]
+    new = x.double() + delta.double().sum(0)
+    ref = P.grouped_rms_norm(new, w.double().cpu(), groups, 1e-5)
+    for out_dtype in (act, torch.float32):
+        xd = x.to(DEV).contiguous()
+        out = torch.empty(T, width, device=DEV, dtype=out_dtype)
+        ops.add_rmsnorm(xd, d_in.to(DEV).contiguous(), w, 1e-5, out, groups=groups)
+        assert rel(xd.double().cpu().numpy(), new.numpy()) < 1e-6
+        assert rel(out.double().cpu().numpy(), ref.numpy()) < (1e-2 if out_dtype == torch.bfloat16 else 1e-5)
+    picked = [T - 2, 0, T - 1]
+    rows = torch.tensor(picked, dtype=torch.int32, device=DEV)
+    some, x_rows = torch.empty(3, width, device=DEV, dtype=act), torch.empty(3, width, device=DEV)
+    ops.add_rmsnorm(x.to(DEV).contiguous(), d_in.to(DEV).contiguous(), w, 1e-5, some, rows, x_rows, groups=groups)
+    assert rel(some.double().cpu().numpy(), ref[picked].numpy()) < (1e-2 if dtype == "bfloat16" else 1e-5)
+    assert rel(x_rows.double().cpu().numpy(), new[picked].numpy()) < 1e-6
+
+
+def test_token_shift_through_its_state():
+    """Portions of one token and of many, two requests side by side in slots that held something else."""
+    from types import SimpleNamespace
+    from rustinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(4)
+    d, lengths = 70, {0: [1, 2, 1, 70, 3, 1, 1, 40], 1: [5, 1, 1, 1, 90, 2, 1, 17]}
+    hs = {r: torch.randn(sum(n), d, generator=g) for r, n in lengths.items()}
+    mix = torch.rand(d, generator=g).to(DEV)
+    state = torch.full((4, d), 9.0, device=DEV)
+    got, pos = {r: [] for r in lengths}, {r: 0 for r in lengths}
+    for step in range(8):
+        ns = [lengths[r][step] for r in lengths]
+        h = torch.cat([hs[r][pos[r]:pos[r] + n] for r, n in zip(lengths, ns)]).to(DEV).contiguous()
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+        ctx = SimpleNamespace(cu_q=i32([0, ns[0], ns[0] + ns[1]]), state_slots=i32([2, 0]), num_rows=2,
+                              positions=i32(list(range(pos[0], pos[0] + ns[0])) + list(range(pos[1], pos[1] + ns[1]))),
+                              row_of_token=i32([0] * ns[0] + [1] * ns[1]))
+        out = torch.empty(sum(ns), d, device=DEV)
+        ops.token_shift(h, mix, state, out, ctx)
+        got[0].append(out[:ns[0]].cpu())
+        got[1].append(out[ns[0]:].cpu())
+        for r, n in zip(lengths, ns):
+            pos[r] += n
+    for r in lengths:
+        ref = P.token_shift(hs[r].double(), mix.double().cpu())
+        assert rel(torch.cat(got[r]).double().numpy(), ref.numpy()) < 1e-6
+    assert float(state[1].min()) == 9.0 and float(state[3].max()) == 9.0      # other requests' slots are left alone
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("decoded", [False, True])
+@pytest.mark.parametrize("window,keep", [(16, 5), (33, 64), (141, 17), (200, 1)])
+def test_keys_at_the_edges_of_window_and_kept_positions_decide(dtype, decoded, window, keep, portion_kernel):
+    """Queries that match one key each, so that the key's weight is near one and all others' near zero: the key
+    that lies window - 1 back is seen and the one that lies window back is not; the last kept position is seen
+    from far away and the position after it is not.  A window or a count of kept positions that is off by
+    one changes these rows beyond any rounding."""
+    T, dk, dv = 460, 16, 12
+    g = torch.Generator().manual_seed(2)
+    eye, look = torch.eye(dk), torch.zeros(dk, dk)          # a query reads feature 8 + n into key feature n
+    q_in, q_out, q_kept, q_lost, q_page = 300, 341, 383, 420, 447
+    marked = {q_in - (window - 1): q_in, q_out - window: q_out, keep - 1: q_kept, keep: q_lost, q_page - window: q_page}
+    x = 0.05 * torch.randn(T, dk, generator=g)
+    x[:, 8:] = 0.0
+    x[:, 14] = 1.0
+    for n, (kpos, qpos) in enumerate(marked.items()):
+        look[n, 8 + n] = 1.0
+        x[kpos] = 0.0
+        x[kpos, n] = 4.0
+        x[qpos, 8 + n] = 4.0
+    x = x.to(torch.bfloat16).float()
+    m = att(1, 1, dk, dv, 30.0 / dk, window, 2, base=100.0, keep=keep)
+    part, pe = attention_part(dk, m, True, eps=1e-6)
+    # rotated features 0, 1 are left out of the match: the keys' own features are 2 .. 6
+    look = torch.roll(look, 2, 0)
+    kmat = torch.roll(eye, 2, 0)
+    wt = {"q": look, "k": kmat, "v": torch.randn(dv, dk, generator=g), "o": torch.randn(dk, dv, generator=g), "pb": torch.tensor([-9.0])}
+    wt = {n: t.to(torch.bfloat16) for n, t in wt.items()}
+    w = load_part(part, wt, dtype)
+    ref = P.sigmoid_attention(x.double(), w, m, 1e-6).numpy()
+    for other in (dict(size=window - 1, keep_first=keep), dict(size=window + 1, keep_first=keep),
+                  dict(size=window, keep_first=keep - 1), dict(size=window, keep_first=keep + 1)):
+        off = P.sigmoid_attention(x.double(), w, dict(m, mask=other), 1e-6).numpy()
+        changed = [q for q in marked.values() if np.abs(ref[q] - off[q]).max() > 0.2 * max(np.abs(ref[q]).max(), np.abs(off[q]).max())]
+        assert len(changed) >= 1, (other, changed)             # the test can tell
+    cuts = [290] + [1] * 170 if decoded else [290, 17, 50, 2, 61, 40]
+    got = run_part(part, [pe], dtype, x, cuts, page=16)
+    scale = np.abs(ref).max()
+    for qpos in marked.values():
+        assert np.abs(got[qpos] - ref[qpos]).max() < PART_TOL[dtype] * scale, qpos
+
+
+# ---------------------------------------------------------------------------
+# whole models
+# ---------------------------------------------------------------------------
+LENGTHS = (70, 3, 121, 1, 38)
+
+
+def test_the_builder_reads_every_tensor(tdirs, plain):
+    from rustinfer_amd.config import load_model_config
+    for name, d in tdirs.items():
+        entry, cfg = load_model_config(d)
+        assert entry.name == "Debuzen"
+        assert set(entry.builder(cfg).param_specs()) == set(plain[name][1])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_every_cut_gives_the_plain_logits(tdirs, plain_logits, name, dtype):
+    reqs, logits = plain_logits(name, LENGTHS, 21)
+    eng = engine_for(tdirs[name], dtype, name)
+    for label, steps in (("whole", cut_whole(reqs)), ("last tokens alone", cut_tail_single(reqs, tail=50)),
+                         ("portions", cut_portions(reqs, seed=3)),
+                         ("portions of two", cut_portions(reqs, seed=4, sizes=(2, 2, 3, 2, 1, 2)))):
+        check_rows(steps, run_steps(eng, steps), logits, dtype, f"{name} {dtype} {label}")
+        assert not eng.cache.live_requests()
+
+
+def test_the_stream_after_every_layer_run(tdirs, plain):
+    """The residual stream after each layer run (a layer of the stretch counts every time) against the plain
+    one: names the first run that differs."""
+    from rustinfer_amd.engine import StepEntry
+    for name in CONFIGS:
+        cfg, w = plain[name]
+        toks = random_requests(cfg["vocab"], (45,), 9)["r0"]
+        want = []
+        P.forward(cfg, w, toks, layers_out=want)
+        eng = engine_for(tdirs[name], "float32", name)
+        got = []
+        for lay in eng.model.layers:
+            def fwd(ctx, hidden, cache, _f=lay.forward, **kw):
+                _f(ctx, hidden, cache, **kw)
+                x = hidden.x.detach().double()
+                if hidden.pending is not None:
+                    x = x + (hidden.pending.double().sum(0) if hidden.pending.dim() == 3 else hidden.pending.double())
+                got.append(x.cpu().numpy().copy())
+            lay.forward = fwd
+        eng.step([StepEntry("r0", toks, list(range(len(toks))))])
+        order = P.run_order(cfg)
+        assert len(got) == len(want) == len(order)
+        for n, (a, b) in enumerate(zip(got, want)):
+            assert rel(a, b.numpy()) < 2e-5, (name, n, order[n], cfg["layers"][order[n][0]]["type"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_mixed_batches_with_pages_and_slots_used_again(tdirs, plain_logits, name, dtype):
+    lengths = (90, 17, 64, 5, 130, 33, 2, 71)
+    reqs, logits = plain_logits(name, lengths, 22)
+    page = PAGE[name]
+    max_tokens = 3 * (-(-130 // 64) * 64)
+    eng = engine_for(tdirs[name], dtype, name, num_pages=max_tokens // page, max_requests=3, max_len=256)
+    steps = cut_mixed(reqs, max_tokens, seed=5, max_live=3, tail=6)
+    assert max(len(st["entries"]) for st in steps) == 3
+    slots, users = set(), {}
+    results = {}
+    from rustinfer_amd.engine import StepEntry
+    for st in steps:
+        lg = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]])
+        slots.update(eng.cache.slot(e["id"]) for e in st["entries"])
+        for e in st["entries"]:
+            for p in eng.cache.table(0, e["id"]):
+                if p >= 0:
+                    users.setdefault(p, set()).add(e["id"])
+        if lg.shape[0]:
+            results[st["step"]] = lg.cpu().numpy()
+        for rid in st["end"]:
+            eng.release(rid)
+    assert len(slots) == 3 and len(reqs) > 3             # eight requests went through three state slots
+    assert any(len(u) > 1 for u in users.values())       # and pages were used again
+    check_rows(steps, results, logits, dtype, f"{name} {dtype} mixed")
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_a_batch_gives_what_each_request_gives_alone(tdirs, name):
+    from rustinfer_amd.engine import StepEntry
+    cfg = CONFIGS[name]
+    reqs = random_requests(cfg["vocab"], (40, 9, 1, 25), 30)
+    eng = engine_for(tdirs[name], "float32", name)
+    alone = {}
+    for rid, toks in reqs.items():
+        if len(toks) > 1:
+            eng.step([StepEntry(rid, toks[:-1], [])])
+        alone[rid] = eng.step([StepEntry(rid, toks[-1:], [0])]).cpu().numpy()[0]
+        eng.release(rid)
+    first = [StepEntry(rid, toks[:-1], []) for rid, toks in reqs.items() if len(toks) > 1]
+    eng.step(first)
+    both = eng.step([StepEntry(rid, toks[-1:], [0]) for rid, toks in reqs.items()]).cpu().numpy()
+    s = float(np.std(both))
+    for row, rid in enumerate(reqs):
+        assert np.abs(both[row] - alone[rid]).max() < 1e-4 * s, rid
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_decoding(tdirs, plain, name):
+    """Twenty tokens of prompt and 280 single tokens: the windows pass over decoded tokens and give their pages
+    back (not those of the kept positions), states, convolution inputs and shifted rows are carried 280 times."""
+    cfg, w = plain[name]
+    toks = random_requests(cfg["vocab"], (300,), 40)["r0"]
+    logits = plain_rows(cfg, w, {"r0": toks})
+    eng = engine_for(tdirs[name], "float32", name, num_pages=40)
+    steps = cut_tail_single({"r0": toks}, tail=280)
+    check_rows(steps, run_steps(eng, steps), logits, "float32", f"{name} long decoding")
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_greedy_generation_through_the_scheduler(tdirs, plain, name):
+    from rustinfer_amd.llm import LLM
+    from rustinfer_amd.sampling import SamplingParams
+    cfg, w = plain[name]
+    prompts = list(random_requests(cfg["vocab"], (12, 47, 5, 30, 21), 50).values())
+    llm = LLM(model=tdirs[name], dtype="float32", paged_block_size=PAGE[name], num_blocks=48, max_batch_seqs=3,
+              max_model_len=128, max_batch_tokens=64, chunked_prefill_size=32)
+    res = llm.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    for p, r in zip(prompts, res):
+        assert len(r.token_ids) == 12
+        toks = list(p)
+        for i, t in enumerate(r.token_ids):
+            row = P.forward(cfg, w, toks)[-1].numpy()
+            assert row.max() - row[t] < 1e-3 * max(1.0, float(np.std(row))), (i, t, int(np.argmax(row)))
+            toks.append(t)
+    assert llm.engine.graph_replays > 0 or not llm.engine._graph_sizes
+
+
+def test_trace_replay_of_a_debuzen_model(tdirs, plain_logits, tmp_path):
+    """bin/trace_run as a user starts it, on the mixed cut, four state slots."""
+    import subprocess
+    import sys
+    from helpers import ROOT
+    name = "A"
+    reqs, logits = plain_logits(name, (50, 20, 9, 77, 30), 60)
+    steps = cut_mixed(reqs, 512, seed=1, max_live=4, tail=5)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", tdirs[name], "--dtype", "bfloat16",
+           "--out", str(tmp_path), "--max-tokens", "512"]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    try:
+        for st in steps:
+            proc.stdin.write(json.dumps(st) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().strip() == f"done {st['step']}"
+        proc.stdin.close()
+        assert proc.wait(timeout=120) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    results = {}
+    for st in steps:
+        n = sum(len(e["want"]) for e in st["entries"])
+        if n:
+            results[st["step"]] = np.fromfile(os.path.join(str(tmp_path), f"{st['step']}.f32"), dtype="<f4").reshape(n, -1)
+    check_rows(steps, results, logits, "bfloat16", "trace replay")
+
+
+# ---------------------------------------------------------------------------
+# configurations drawn at random
+# ---------------------------------------------------------------------------
+def draw_config(rng):
+    """A configuration whose every size, the order of its layers, the norm's groups and its stretch are drawn:
+    widths up to 768, up to 16 heads, windows and kept positions around page borders, convolutions of 1 to 8
+    taps, layers without feed-forward, a stretch anywhere or none."""
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+
+    def left(sigmoid):
+        H = pick([1, 2, 4, 6, 8, 12, 16])
+        d = pick([16, 32, 48, 64, 96, 128])
+        return att(H, pick([g for g in (1, 2, 3, 4, 8) if H % g == 0]), d, pick([16, 32, 64, 96, 128]), pick([0.1, 0.125, 0.2]),
+                   pick([5, 16, 17, 48, 100, 128, 150, 256]), pick([r for r in (4, 16, 32, 48, 64) if r <= d]), base=pick([100.0, 1e4, 1e6]),
+                   keep=pick([0, 1, 6, 16, 17, 70]) if sigmoid else None)
+
+    layers = []
+    for _ in range(int(rng.integers(3, 8))):
+        k = rng.random()
+        if k < 0.3:
+            mixer = gla(pick([1, 2, 4, 6, 8]), pick([16, 32, 64, 128]), pick([16, 32, 64, 128]), pick([1.0, 4.0, 16.0]))
+        elif k < 0.65:
+            H = pick([1, 2, 4, 6, 8, 12])
+            mixer = par(left(True), H, pick([g for g in (1, 2, 3, 4, 6) if H % g == 0]), pick([16, 32, 64, 96, 128]), pick([16, 32, 64, 128]),
+                        pick([1, 2, 3, 4, 5, 8]), ls=pick([0.5, 0.6, 1.0, 1.2]), rs=pick([0.5, 1.0, 1.5]))
+        else:
+            H, dv = pick([2, 4, 6, 8, 12]), pick([16, 32, 64])
+            mixer = par2(left(False), H, dv, pick([16, 48, 64, 128]), pick([g for g in (1, 2, 3, 4) if H % g == 0]), pick([1, 2, 3, 4, 8]),
+                         pick([g for g in (1, 2, 4) if (H * dv) % g == 0]), ls=pick([0.5, 0.6, 1.0, 1.2]), rs=pick([0.5, 1.0, 1.5]))
+        layers.append(layer(mixer, None if rng.random() < 0.15 else pick([64, 200, 512, 1024])))
+    width = pick([64, 96, 192, 320, 768])
+    cfg = dict(architecture="Debuzen", vocab=pick([100, 333, 777, 1000]), width=width,
+               norm=dict(eps=pick([1e-5, 1e-6]), groups=pick([g for g in (1, 2, 3, 4, 8) if width % g == 0])),
+               logit_softcap=pick([0.0, 15.0, 30.0]), layers=layers)
+    if rng.random() < 0.75:
+        a = int(rng.integers(0, len(layers)))
+        cfg["loop"] = dict(start=a, stop=int(rng.integers(a + 1, len(layers) + 1)), times=int(rng.integers(1, 4)))
+    return cfg
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15, 16])
+def test_configurations_drawn_at_random(seed, tmp_path):
+    """In 32-bit, where rounding hides nothing: last tokens alone, portions, and a mixed schedule on a pool
+    that is too small for all requests at once, against the plain implementation."""
+    from rustinfer_amd.engine import build_engine
+    from rustinfer_amd.weights import write_safetensors
+    cfg = draw_config(np.random.default_rng(seed))
+    w = draw_weights(cfg, seed)
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(cfg, f)
+    write_safetensors(str(tmp_path / "model.safetensors"), w)
+    reqs = random_requests(cfg["vocab"], (150, 3, 290, 40, 1, 77), seed)
+    logits = Rows({rid: P.forward(cfg, w, toks).numpy() for rid, toks in reqs.items()})
+    max_tokens = 2 * 320 + 64
+    eng = build_engine(str(tmp_path), dtype="float32", device=DEV, page_size=16, num_pages=max_tokens // 16, max_requests=4,
+                       max_model_len=max_tokens, max_batch_tokens=2048)
+    for label, steps in (("last tokens alone", cut_tail_single(reqs, tail=40)), ("portions", cut_portions(reqs, seed=seed)),
+                         ("mixed", cut_mixed(reqs, max_tokens, seed=seed, max_live=4, tail=6))):
+        check_rows(steps, run_steps(eng, steps), logits, "float32", f"{json.dumps(cfg)} {label}")
+        assert not eng.cache.live_requests()
