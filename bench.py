@@ -542,20 +542,87 @@ def _count(shape):
     return n
 
 
+# Debuzen at the layer sizes of the Llama shapes: the same width, feed-forward width and heads.  Its mixers take
+# turns; a mixer of two halves gives each half of the shape's heads (attention in a window of 1,024 positions,
+# four kept first positions where the design has them; the delta rule on heads of the shape's size with
+# convolutions of four taps; the state-space half on a state of two head sizes a head); gated linear attention
+# has all the heads.  Layers 2 and 3 run twice, as in the Pilavik model it stands beside.
+DEBUZEN_PATTERN = ("parallel_2", "gla", "parallel")
+
+
+def debuzen_config(shape_name, layers=0, window=1024):
+    s = SHAPES[shape_name]
+    H, G, hd, W, ff = s["num_attention_heads"], s["num_key_value_heads"], s["head_dim"], s["hidden_size"], s["intermediate_size"]
+    runs = layers or s["num_hidden_layers"]
+    loop = dict(start=2, stop=4, times=2) if runs >= 6 else None
+    h2, g2 = max(H // 2, 1), max(G // 2, 1)
+    out = []
+    for i in range(runs - 2 if loop else runs):
+        kind = DEBUZEN_PATTERN[i % len(DEBUZEN_PATTERN)]
+        left = dict(heads=h2, kv_heads=g2, dim=hd, vdim=hd, scale=hd ** -0.5, mask=dict(size=window), rot=dict(base=10000.0, dims=hd // 2))
+        if kind == "gla":
+            mixer = dict(heads=H, dim=hd, vdim=hd, tau=16.0, decay_rank=16)
+        elif kind == "parallel":
+            left["mask"]["keep_first"] = 4
+            mixer = dict(left=left, right=dict(heads=h2, kv_heads=g2, dim=hd, vdim=hd, conv=4, decay_rank=32, gate_rank=32),
+                         left_scale=1.0, right_scale=0.5)
+        else:
+            mixer = dict(left=left, right=dict(heads=h2, vdim=hd, state=2 * hd, groups=g2, conv=4, norm_groups=g2),
+                         left_scale=0.6, right_scale=0.5)
+        out.append(dict(type=kind, mixer=mixer, mlp=dict(kind="dense", ff=ff)))
+    conf = dict(architecture="Debuzen", vocab=s["vocab_size"], width=W, norm=dict(eps=1e-6, groups=4), logit_softcap=30.0, layers=out)
+    if loop:
+        conf["loop"] = loop
+    return conf
+
+
+class DebuzenBench(TedelixBench):
+    """The same measurements on a Debuzen model of a Llama shape's sizes."""
+
+    def design_config(self, shape_name, args):
+        return debuzen_config(shape_name, args.layers, self.window)
+
+    def account(self, cfg, el):
+        # every layer RUN reads its weights, its window of keys and values and its states: a layer of the stretch counts `times` times
+        self.window_kv_bytes = self.state_bytes = 0
+        self.attn_flops_per_key = self.scan_flops_per_token = 0
+        again = 0
+        for i, layer in enumerate(cfg.layers):
+            times = cfg.loop_times if cfg.has_loop and cfg.loop_start <= i < cfg.loop_stop else 1
+            m = layer.mixer
+            if layer.type == "gla":
+                self.state_bytes += times * 2 * 4 * m.heads * m.dim * m.vdim
+                self.scan_flops_per_token += times * 2.0 * 2 * m.heads * m.dim * m.vdim
+            else:
+                a, r = m.left, m.right
+                self.window_kv_bytes += times * a.kv_heads * (a.dim + a.vdim) * el
+                self.attn_flops_per_key += times * 2.0 * a.heads * (a.dim + a.vdim)
+                rows = r.dim if layer.type == "parallel" else r.state
+                self.state_bytes += times * 2 * 4 * r.heads * rows * r.vdim
+                self.scan_flops_per_token += times * 2.0 * (4 if layer.type == "parallel" else 2) * r.heads * rows * r.vdim
+            if times > 1:
+                again += (times - 1) * sum(_count(spec.shape) for name, spec in self.engine.model.param_specs().items()
+                                           if name.startswith(f"l{i}."))
+        if cfg.has_loop:
+            again += (cfg.loop_times - 1) * 2 * cfg.hidden_size * cfg.hidden_size      # the product in front of every pass
+        self.params += again                      # weights read (and multiplied) a step, not weights stored
+        self.weight_bytes = el * self.params
+
+
 DESIGNS = {"tedelix": (TedelixBench, "llama", TEDELIX_PATTERN), "belorax": (BeloraxBench, "tedelix", BELORAX_PATTERN),
-           "pilavik": (PilavikBench, "belorax", PILAVIK_PATTERN)}
+           "pilavik": (PilavikBench, "belorax", PILAVIK_PATTERN), "debuzen": (DebuzenBench, "pilavik", DEBUZEN_PATTERN)}
 
 
 def design_record(args, peaks):
-    """``--design tedelix|belorax|pilavik``: decode at the main batch and prefill of 2,048 tokens for models
-    of that design at the sizes of ``--design-shapes``, each beside the closest other design at the same
-    sizes (Tedelix beside Llama, Belorax beside Tedelix, Pilavik beside Belorax)."""
+    """``--design tedelix|belorax|pilavik|debuzen``: decode at the main batch and prefill of 2,048 tokens for
+    models of that design at the sizes of ``--design-shapes``, each beside the closest other design at the same
+    sizes (Tedelix beside Llama, Belorax beside Tedelix, Pilavik beside Belorax, Debuzen beside Pilavik)."""
     design_cls, beside, pattern = DESIGNS[args.design]
-    others = {"llama": Bench, "tedelix": TedelixBench, "belorax": BeloraxBench}
+    others = {"llama": Bench, "tedelix": TedelixBench, "belorax": BeloraxBench, "pilavik": PilavikBench}
     out = {"metric": "decode tok/s at batch %d and prefill tok/s at 2,048 tokens: %s beside %s at equal layer sizes" % (args.batch, args.design, beside),
            "unit": "tok/s", "dtype": args.dtype, "data": "synthetic: random weights, random token ids", "peaks": peaks,
            "pattern": list(pattern), "shapes": {}}
-    if args.design in ("tedelix", "pilavik"):
+    if args.design in ("tedelix", "pilavik", "debuzen"):
         out["window"] = 1024
     steps = max(MIN_POINT_STEPS, args.steps)
     for name in args.design_shapes.split(","):
@@ -652,8 +719,8 @@ def main() -> int:
                     help="only time the sampling kernels on 1, 8 and 64 rows of the shape's vocabulary")
     ap.add_argument("--no-gemm-tune", action="store_true",
                     help="keep the GEMM library's own choice of kernel for the prompt's products")
-    ap.add_argument("--design", default="llama", choices=["llama", "tedelix", "belorax", "pilavik"],
-                    help="tedelix, belorax, pilavik: only decode and prefill of models of that design at the sizes of "
+    ap.add_argument("--design", default="llama", choices=["llama", "tedelix", "belorax", "pilavik", "debuzen"],
+                    help="tedelix, belorax, pilavik, debuzen: only decode and prefill of models of that design at the sizes of "
                          "--design-shapes, each beside the closest other design at the same sizes (Tedelix beside Llama, "
                          "Belorax beside Tedelix, Pilavik beside Belorax; the default workload is not run)")
     ap.add_argument("--design-shapes", default="1b,3b", help="shapes for --design other than llama, with commas between them")

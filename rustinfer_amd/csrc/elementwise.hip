@@ -53,12 +53,22 @@ extern "C" int ri_embed(const int* ids, const int* device_tokens, const void* ta
 // delta may be a stack of `parts` 32-bit partial sums (what a product split over K leaves).
 // VEC elements per thread and load: 4 when d % 4 == 0, else 1.
 // ---------------------------------------------------------------------------
+// A token shift on the normed rows, for steps whose every row is one token (row b is token b): the row leaves
+// as y + (prev - y) * mix with prev the request's last normed row from state [slots][row width] (zeros at position
+// 0), and y takes its place there.  mix null: none.
+struct NormShift {
+    const float* mix;
+    float* state;
+    const int* slots;
+    const int* positions;
+};
+
 // PARTS > 0: that many partial sums, all requested before any is added; 0: a runtime count.
 template <typename TD, typename TW, typename TO, int BLOCK, int VEC, int PARTS>
 __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
         float* __restrict__ x, const TD* __restrict__ delta, int parts_rt, size_t part_stride,
         const TW* __restrict__ w_all, TO* __restrict__ out, int d, float eps, const int* __restrict__ rows,
-        float* __restrict__ x_rows, int groups) {
+        float* __restrict__ x_rows, int groups, const NormShift sh) {
     __shared__ float red[16];
     using L = VecLoad<VEC>;
     // groups > 1: a row is `groups` consecutive parts of d values, each normed by itself: a block a part
@@ -125,6 +135,17 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
     }
     ss = block_sum(ss, red);
     const float rs = rsqrtf(ss / (float)d + eps);
+    float* st = sh.mix ? sh.state + ((size_t)sh.slots[tok] * groups + part) * d : nullptr;
+    const float* mixp = sh.mix ? sh.mix + (size_t)part * d : nullptr;
+    const bool has_prev = sh.mix && sh.positions[tok] > 0;
+    auto shifted = [&](int i, float* y) {
+        float pv[VEC], mx[VEC];
+        L::ld(st + i, pv);
+        L::ld(mixp + i, mx);
+        L::st(st + i, y);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) y[e] = fmaf((has_prev ? pv[e] : 0.f) - y[e], mx[e], y[e]);
+    };
 #pragma unroll
     for (int k = 0; k < CACHE; ++k) {
         const int i = (threadIdx.x + k * BLOCK) * VEC;
@@ -132,6 +153,7 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
             float y[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) y[e] = v[k][e] * rs * wv[k][e];
+            if (st) shifted(i, y);
             L::st(o + i, y);
         }
     }
@@ -149,14 +171,16 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
         L::ld(w + i, ww);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) y[e] = a[e] * rs * ww[e];
+        if (st) shifted(i, y);
         L::st(o + i, y);
     }
 }
 
 template <typename TD, typename TW, typename TO>
 static int launch_add_rmsnorm(float* x, const void* delta, int parts, size_t part_stride, const void* w,
-                              void* out, int n_out, int d, float eps, const int* rows, float* x_rows, int groups, hipStream_t stream) {
-#define RI_NORM_ARGS x, (const TD*)delta, parts, part_stride, (const TW*)w, (TO*)out, d, eps, rows, x_rows, groups
+                              void* out, int n_out, int d, float eps, const int* rows, float* x_rows, int groups, hipStream_t stream,
+                              NormShift sh = NormShift{nullptr, nullptr, nullptr, nullptr}) {
+#define RI_NORM_ARGS x, (const TD*)delta, parts, part_stride, (const TW*)w, (TO*)out, d, eps, rows, x_rows, groups, sh
 #define RI_NORM_LAUNCH(BLOCK, VEC) do { \
         if (parts == 1) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 1><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
         else if (parts == 2) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 2><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
@@ -212,6 +236,31 @@ extern "C" int ri_add_rmsnorm(float* x, const void* delta, int delta_dtype, int 
     if (delta_dtype == RI_BF16 && w_dtype == RI_F32 && out_dtype == RI_F32) return launch_add_rmsnorm<bf16_t, float, float>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, groups, stream);
     if (delta_dtype == RI_F32 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, groups, stream);
     return ri_fail("ri_add_rmsnorm: unsupported dtypes delta=%d weight=%d out=%d", delta_dtype, w_dtype, out_dtype);
+}
+
+// ri_add_rmsnorm for a step whose every row is one token, with a token shift on the normed rows (see NormShift):
+// mix [d] and state [slots][d] 32-bit, slots and positions one a row.  The 32-bit weight only.
+extern "C" int ri_add_rmsnorm_shift(float* x, const void* delta, int delta_dtype, int parts, long long part_stride,
+                                    const float* w, void* out, int out_dtype, int T, int d, float eps, int groups,
+                                    const float* mix, float* state, int num_slots, const int* slots, const int* positions,
+                                    hipStream_t stream) {
+    RI_REQUIRE(T >= 0 && d > 0 && groups >= 1 && d % groups == 0 && num_slots > 0, "ri_add_rmsnorm_shift: bad sizes T=%d d=%d groups=%d", T, d, groups);
+    RI_REQUIRE(eps > 0.f, "ri_add_rmsnorm_shift: eps must be > 0");
+    RI_REQUIRE(!delta || (parts >= 1 && part_stride >= 0), "ri_add_rmsnorm_shift: bad parts");
+    if (T == 0) return 0;
+    RI_REQUIRE(x && w && out && mix && state && slots && positions, "ri_add_rmsnorm_shift: null pointer");
+    RI_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)delta % 16 == 0
+               && (uintptr_t)mix % 16 == 0 && (uintptr_t)state % 16 == 0, "ri_add_rmsnorm_shift: operands must be 16-byte aligned");
+    RI_REQUIRE((long long)T * groups <= 2147483647LL, "ri_add_rmsnorm_shift: too many rows for the grid");
+    const int dg = d / groups, n_out = T * groups;
+    RI_REQUIRE(dg % 4 != 0 || part_stride % 4 == 0, "ri_add_rmsnorm_shift: part stride must be a multiple of 4");
+    if (!delta) delta_dtype = RI_F32;
+    const size_t ps = (size_t)part_stride;
+    const NormShift sh{mix, state, slots, positions};
+    if (delta_dtype == RI_F32 && out_dtype == RI_F32) return launch_add_rmsnorm<float, float, float>(x, delta, parts, ps, w, out, n_out, dg, eps, nullptr, nullptr, groups, stream, sh);
+    if (delta_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, float, bf16_t>(x, delta, parts, ps, w, out, n_out, dg, eps, nullptr, nullptr, groups, stream, sh);
+    if (delta_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, float, bf16_t>(x, delta, parts, ps, w, out, n_out, dg, eps, nullptr, nullptr, groups, stream, sh);
+    return ri_fail("ri_add_rmsnorm_shift: unsupported dtypes delta=%d out=%d", delta_dtype, out_dtype);
 }
 
 // ---------------------------------------------------------------------------

@@ -192,6 +192,39 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
                                  _ptr(rows), _ptr(x_rows), int(groups), _stream()))
 
 
+def add_rmsnorm_shift(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float, out: torch.Tensor,
+                      mix: torch.Tensor, state: torch.Tensor, ctx, groups: int = 1) -> None:
+    """``add_rmsnorm`` and ``token_shift`` in one pass, for a step whose every row is one token (row b is token
+    b): ``x += delta``, ``h = rmsnorm(x) * weight`` (in ``groups`` parts), ``out = h + (prev - h) * mix`` with
+    ``prev`` the request's last ``h`` from ``state [slots, d]`` (zeros at position 0), which ``h`` replaces.
+    ``weight``, ``mix`` and ``state`` 32-bit."""
+    _dev(x, delta, weight, out, mix, state)
+    T, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or tuple(out.shape) != (T, d) or not out.is_contiguous():
+        raise KernelError("add_rmsnorm_shift: contiguous float32 x [T, d] and contiguous out [T, d] expected")
+    if T > ctx.num_rows or ctx.max_q_len != 1:
+        raise KernelError("add_rmsnorm_shift: only for steps whose every row is one token")
+    parts, stride, ddt = 1, 0, F32
+    if delta is not None:
+        if delta.dim() == 3:
+            parts, stride = delta.shape[0], delta.stride(0)
+        if delta.dim() not in (2, 3) or tuple(delta.shape[-2:]) != (T, d) or delta.stride(-1) != 1 or delta.stride(-2) != d \
+                or (delta.dim() == 3 and delta.dtype != torch.float32):
+            raise KernelError("add_rmsnorm_shift: delta must be [T, d] or a float32 stack [P, T, d] with contiguous rows")
+        ddt = _dt(delta)
+    _f32_vec(weight, d, "add_rmsnorm_shift: the weight")
+    _f32_vec(mix, d, "add_rmsnorm_shift: the mixing weights")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != d or not state.is_contiguous():
+        raise KernelError(f"add_rmsnorm_shift: state must be contiguous float32 [slots, {d}]")
+    if groups < 1 or d % groups:
+        raise KernelError(f"add_rmsnorm_shift: {d} values do not split into {groups} equal parts")
+    _i32(ctx.positions, "positions", T)
+    _i32(ctx.state_slots, "state_slots", ctx.num_rows)
+    _check(_lib().ri_add_rmsnorm_shift(_ptr(x), _ptr(delta), ddt, parts, ctypes.c_longlong(stride), _ptr(weight), _ptr(out),
+                                       _dt(out), T, d, ctypes.c_float(eps), int(groups), _ptr(mix), _ptr(state), state.shape[0],
+                                       _ptr(ctx.state_slots), _ptr(ctx.positions), _stream()))
+
+
 def _check_cache(k_cache, v_cache, Hkv, hd, page, act_dtype, name):
     if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (Hkv, page, hd) or v_cache.dim() != 4 \
             or tuple(v_cache.shape) != (k_cache.shape[0], Hkv, hd, page):

@@ -142,6 +142,13 @@ class PreNormBlock(Part):
         leaves 32-bit rows, and the shift rounds once)."""
         if self.mixer_shift is None:
             return hidden.input_behind(ctx, self.mixer_norm, normed)
+        fused = getattr(self.mixer_norm, "forward_shifted", None)
+        if fused is not None and ctx.max_q_len == 1 and normed.shape[0] <= ctx.num_rows:
+            # every row is one token: norm and shift are one kernel (the previous rows come from the slots alone)
+            hidden.deferred = None
+            fused(ctx, hidden.x, hidden.pending, normed, self.mixer_shift.mix, self.mixer_shift.state_of(cache))
+            hidden.pending = None
+            return normed
         h32 = ctx.workspace.get("block.normed32", normed.shape[0], self.hidden_size, torch.float32)
         hidden.deferred = None
         self.mixer_norm.forward(ctx, hidden.x, hidden.pending, h32)

@@ -61,6 +61,15 @@ class RMSNorm(Norm):
         return out
 
 
+    def forward_shifted(self, ctx, x, delta, out, mix, state):
+        """For a step whose every row is one token: ``forward`` and a token shift on what it leaves (``mix``, and
+        the requests' last normed rows in ``state``), in one kernel."""
+        if self.weight.dtype != torch.float32:
+            raise RuntimeError("the norm in front of a token shift keeps its weight in 32-bit (weight_32bit=True)")
+        self.rt.ops.add_rmsnorm_shift(x, delta, self.weight, self.eps, out, mix, state, ctx, groups=self.groups)
+        return out
+
+
 class OutputRMSNorm(Norm):
     """The norm of a block whose sub-layers read the residual stream itself: it sits on a sub-layer's
     OUTPUT, and what it leaves is added to the stream, ``x += mult * y * rsqrt(mean(y^2) + eps) * w``

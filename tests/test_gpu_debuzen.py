@@ -374,6 +374,43 @@ def test_token_shift_through_its_state():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width,groups,parts", [(64, 4, 1), (100, 5, 3), (4096, 2, 8), (33, 3, 1), (18, 1, 2)])
+def test_norm_and_shift_in_one_pass_for_single_tokens(dtype, width, groups, parts):
+    """Steps whose every row is one token: the same bits as the norm's kernel followed by the shift's, row after
+    row through the slots, and the plain result."""
+    from types import SimpleNamespace
+    from rustinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(width + parts)
+    act = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    B, steps = 3, 5
+    xs = torch.randn(steps, B, width, generator=g) * 2.0
+    deltas = torch.randn(steps, parts, B, width, generator=g)
+    w = (1.0 + 0.3 * torch.randn(width, generator=g)).to(DEV)
+    mix = torch.rand(width, generator=g).to(DEV)
+    one, two = torch.full((5, width), 7.0, device=DEV), torch.full((5, width), 7.0, device=DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    outs = []
+    for t in range(steps):
+        ctx = SimpleNamespace(cu_q=i32([0, 1, 2, 3]), state_slots=i32([4, 0, 2]), num_rows=B, max_q_len=1,
+                              positions=i32([t, t, t]), row_of_token=i32([0, 1, 2]))
+        d_in = (deltas[t] if parts > 1 else deltas[t, 0]).to(DEV).contiguous()
+        xa, xb = xs[t].to(DEV).contiguous(), xs[t].to(DEV).contiguous()
+        fused = torch.empty(B, width, device=DEV, dtype=act)
+        ops.add_rmsnorm_shift(xa, d_in, w, 1e-5, fused, mix, one, ctx, groups=groups)
+        h32, apart = torch.empty(B, width, device=DEV), torch.empty(B, width, device=DEV, dtype=act)
+        ops.add_rmsnorm(xb, d_in, w, 1e-5, h32, groups=groups)
+        ops.token_shift(h32, mix, two, apart, ctx)
+        assert torch.equal(fused, apart) and torch.equal(one, two) and torch.equal(xa, xb)
+        outs.append(fused.double().cpu())
+    h = P.grouped_rms_norm((xs.double() + deltas.double().sum(1)).reshape(steps * B, width), w.double().cpu(), groups, 1e-5).reshape(steps, B, width)
+    for b in range(B):
+        ref = P.token_shift(h[:, b], mix.double().cpu())
+        got = torch.stack([o[b] for o in outs])
+        assert rel(got.numpy(), ref.numpy()) < (1e-2 if dtype == "bfloat16" else 1e-5)
+    assert float(one[1].min()) == 7.0 and float(one[3].max()) == 7.0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("decoded", [False, True])
 @pytest.mark.parametrize("window,keep", [(16, 5), (33, 64), (141, 17), (200, 1)])
 def test_keys_at_the_edges_of_window_and_kept_positions_decide(dtype, decoded, window, keep, portion_kernel):
