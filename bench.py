@@ -545,7 +545,7 @@ def _count(shape):
 # Debuzen at the layer sizes of the Llama shapes: the same width, feed-forward width and heads.  Its mixers take
 # turns; a mixer of two halves gives each half of the shape's heads (attention in a window of 1,024 positions,
 # four kept first positions where the design has them; the delta rule on heads of the shape's size with
-# convolutions of four taps; the state-space half on a state of two head sizes a head); gated linear attention
+# convolutions of four taps; the state-space half on a state of 128 rows a head); gated linear attention
 # has all the heads.  Layers 2 and 3 run twice, as in the Pilavik model it stands beside.
 DEBUZEN_PATTERN = ("parallel_2", "gla", "parallel")
 
@@ -567,7 +567,7 @@ def debuzen_config(shape_name, layers=0, window=1024):
             mixer = dict(left=left, right=dict(heads=h2, kv_heads=g2, dim=hd, vdim=hd, conv=4, decay_rank=32, gate_rank=32),
                          left_scale=1.0, right_scale=0.5)
         else:
-            mixer = dict(left=left, right=dict(heads=h2, vdim=hd, state=2 * hd, groups=g2, conv=4, norm_groups=g2),
+            mixer = dict(left=left, right=dict(heads=h2, vdim=hd, state=128, groups=g2, conv=4, norm_groups=g2),
                          left_scale=0.6, right_scale=0.5)
         out.append(dict(type=kind, mixer=mixer, mlp=dict(kind="dense", ff=ff)))
     conf = dict(architecture="Debuzen", vocab=s["vocab_size"], width=W, norm=dict(eps=1e-6, groups=4), logit_softcap=30.0, layers=out)

@@ -36,21 +36,37 @@ __global__ __launch_bounds__(256) void token_shift_kernel(
     }
 }
 
-template <typename TD, typename TY, typename TO>
+// VEC values a thread (4 where the row length, the parts' stride and every pointer allow 16-byte loads of 32-bit
+// values); a row is dealt to several blocks, and up to eight partial sums are asked for before any is added.
+template <typename TD, typename TY, typename TO, int VEC>
 __global__ __launch_bounds__(256) void stream_pair_kernel(
         const float* __restrict__ x, const TD* __restrict__ delta, int parts, size_t part_stride,
         const TY* __restrict__ y, TO* __restrict__ out, int d) {
+    using L = VecLoad<VEC>;
     const int t = blockIdx.x;
-    const float* xr = x + (size_t)t * d;
-    const TY* yr = y + (size_t)t * d;
-    TO* o = out + (size_t)t * 2 * d;
-    for (int c = threadIdx.x; c < d; c += 256) {
-        float v = xr[c];
-        if (delta)
-            for (int p = 0; p < parts; ++p) v += ld_f32(delta + p * part_stride + (size_t)t * d + c);
-        st_f32(o + c, v);
-        st_f32(o + d + c, ld_f32(yr + c));
+    const int c = ((int)blockIdx.y * 256 + threadIdx.x) * VEC;
+    if (c >= d) return;
+    const size_t at = (size_t)t * d + c;
+    float v[VEC], yv[VEC];
+    L::ld(x + at, v);
+    L::ld(y + at, yv);
+    if (delta) {
+        for (int p0 = 0; p0 < parts; p0 += 8) {
+            float part[8][VEC];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (p0 + i < parts) L::ld(delta + (size_t)(p0 + i) * part_stride + at, part[i]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (p0 + i < parts) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) v[e] += part[i][e];
+                }
+        }
     }
+    TO* o = out + (size_t)t * 2 * d;
+    L::st(o + c, v);
+    L::st(o + d + c, yv);
 }
 
 }  // namespace
@@ -78,7 +94,11 @@ extern "C" int ri_stream_pair(const float* x, const void* delta, int delta_dtype
     if (T == 0) return 0;
     RI_REQUIRE(x && y && out, "ri_stream_pair: null pointer");
     const size_t ps = (size_t)part_stride;
-#define RI_PAIR(TD, TY, TO) stream_pair_kernel<TD, TY, TO><<<T, 256, 0, stream>>>(x, (const TD*)delta, parts, ps, (const TY*)y, (TO*)out, d)
+    const bool vec = d % 4 == 0 && part_stride % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0 && (uintptr_t)delta % 16 == 0
+                     && (uintptr_t)out % 16 == 0;
+    const dim3 grid(T, vec ? (d / 4 + 255) / 256 : (d + 255) / 256);
+#define RI_PAIR(TD, TY, TO) do { if (vec) stream_pair_kernel<TD, TY, TO, 4><<<grid, 256, 0, stream>>>(x, (const TD*)delta, parts, ps, (const TY*)y, (TO*)out, d); \
+        else stream_pair_kernel<TD, TY, TO, 1><<<grid, 256, 0, stream>>>(x, (const TD*)delta, parts, ps, (const TY*)y, (TO*)out, d); } while (0)
     if (!delta) delta_dtype = RI_F32;
     if (delta_dtype == RI_F32 && y_dtype == RI_F32 && out_dtype == RI_F32) RI_PAIR(float, float, float);
     else if (delta_dtype == RI_F32 && y_dtype == RI_F32 && out_dtype == RI_BF16) RI_PAIR(float, float, bf16_t);
