@@ -1038,7 +1038,8 @@ class StateSpaceSpec:
 class TwoMixerSpec:
     """Mixers ``parallel`` (attention with sigmoid weights and kept first positions beside the channel-gated
     delta rule) and ``parallel_2`` (softmax attention with a sink beside a state-space mixer): both halves read
-    the same rows, and the result is ``left_scale * left + right_scale * right``."""
+    the same rows, and the result is ``left_scale * left + right_scale * right``.  A mask's ``keep_first`` is
+    honoured in either (absent: none)."""
     kind: str
     left: MaskedAttentionSpec
     right: Any
@@ -1051,8 +1052,6 @@ class TwoMixerSpec:
         s = TwoMixerSpec(kind, MaskedAttentionSpec.from_dict(_obj(m, "left", where), where + ".left"),
                          right_cls.from_dict(_obj(m, "right", where), where + ".right"),
                          _require(m, "left_scale", float, where), _require(m, "right_scale", float, where))
-        if kind == "parallel_2" and s.left.keep_first:
-            raise ConfigError(f"{where}.left.mask: the softmax half keeps no first positions")
         return s
 
     def to_dict(self) -> Dict[str, Any]:

@@ -75,7 +75,7 @@ def build_debuzen(cfg: DebuzenConfig) -> DecoderModel:
     def attention(a, sigmoid: bool):
         return WindowAttention(width, a.heads, a.kv_heads, a.dim, a.vdim, a.scale, window=a.window,
                                pos_enc=rotation(a.dim, a.rot_base, a.rot_dims), interleaved=sigmoid,
-                               qk_unit_eps=eps if sigmoid else None, keep_first=a.keep_first if sigmoid else 0,
+                               qk_unit_eps=eps if sigmoid else None, keep_first=a.keep_first,
                                sink=not sigmoid, sigmoid_weights=sigmoid)
 
     layers = []

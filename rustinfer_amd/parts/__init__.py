@@ -12,3 +12,5 @@ from .block import Hidden, ParallelBlock, PostNormBlock, PreNormBlock, SandwichB
 from .registry import (MIXERS, FEED_FORWARDS, NORMS, POSITION_ENCODINGS, register_mixer,
                        register_feed_forward, register_norm, register_position_encoding,
                        make_part)
+
+register_mixer("two_mixers", TwoMixers)

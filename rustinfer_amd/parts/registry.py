@@ -7,12 +7,15 @@ from typing import Callable, Dict
 from .attention import LatentAttention, PagedAttention, WindowAttention
 from .mlp import DenseMLP, MoEFeedForward, PolyNormMLP, SwiGLUMLP
 from .norm import LayerNorm, OutputRMSNorm, RMSNorm
-from .recurrent import GatedDeltaRule, GeneralDeltaRule, LightningAttention, Retention
+from .recurrent import (ChannelGatedDeltaRule, GatedDeltaRule, GatedLinearAttention, GeneralDeltaRule, LightningAttention,
+                        Retention, StateSpaceMixer)
 from .rope import RotaryEmbedding
 
 MIXERS: Dict[str, Callable] = {"attention": PagedAttention, "window_attention": WindowAttention,
                                "lightning": LightningAttention, "general_delta": GeneralDeltaRule,
-                               "latent_attention": LatentAttention, "retention": Retention, "gated_delta": GatedDeltaRule}
+                               "latent_attention": LatentAttention, "retention": Retention, "gated_delta": GatedDeltaRule,
+                               "channel_gated_delta": ChannelGatedDeltaRule, "gated_linear_attention": GatedLinearAttention,
+                               "state_space": StateSpaceMixer}
 FEED_FORWARDS: Dict[str, Callable] = {"swiglu": SwiGLUMLP, "dense": DenseMLP, "moe": MoEFeedForward, "poly_norm": PolyNormMLP}
 NORMS: Dict[str, Callable] = {"rmsnorm": RMSNorm, "output_rmsnorm": OutputRMSNorm, "layernorm": LayerNorm}
 POSITION_ENCODINGS: Dict[str, Callable] = {"rope": RotaryEmbedding}

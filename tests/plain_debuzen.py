@@ -105,7 +105,7 @@ def sink_attention(h, W, m):
     q = rotate(q, m["rot"]["base"], m["rot"]["dims"], False)
     k = rotate(k, m["rot"]["base"], m["rot"]["dims"], False)
     s = windowed_scores(q, k, m["scale"], H, G)
-    see = visible(T, m["mask"]["size"])
+    see = visible(T, m["mask"]["size"], m["mask"].get("keep_first", 0))
     s = s.masked_fill(~see[None], -math.inf)
     sink = W["sink"][:, None, None].expand(H, T, 1)
     p = torch.softmax(torch.cat([s, sink], dim=-1), dim=-1)[..., :T]

@@ -61,7 +61,7 @@ def test_reads_every_size_and_constant():
     ((("layers", 0, "type"), "attention"), "unknown mixer"), ((("layers", 1, "mixer", "right", "kv_heads"), 3), "multiple"),
     ((("layers", 1, "mixer", "right", "conv"), 0), "> 0"), ((("layers", 1, "mixer", "left", "rot", "dims"), 12), "rot.dims"),
     ((("layers", 1, "mixer", "left", "mask", "size"), 0), "size"), ((("layers", 2, "mixer", "left", "scale"), KeyError), "scale"),
-    ((("layers", 2, "mixer", "left", "mask", "keep_first"), 4), "keeps no first"), ((("layers", 2, "mixer", "right", "groups"), 3), "groups"),
+    ((("layers", 2, "mixer", "left", "mask", "keep_first"), -1), "keep_first"), ((("layers", 2, "mixer", "right", "groups"), 3), "groups"),
     ((("layers", 2, "mixer", "left_scale"), KeyError), "left_scale"), ((("layers", 0, "mixer", "tau"), 0.0), "tau"),
     ((("layers", 0, "mlp", "kind"), "sparse"), "kind"), ((("layers", 0, "mlp", "ff"), 0), "ff"), ((("loop", "stop"), 5), "stop"),
     ((("loop", "times"), 0), "times"), ((("width",), KeyError), "width"), ((("norm", "eps"), 0.0), "eps"),

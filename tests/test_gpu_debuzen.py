@@ -195,7 +195,7 @@ def attention_part(width, m, sigmoid, eps=1e-5):
     from rustinfer_amd.parts import RotaryEmbedding, WindowAttention
     pe = RotaryEmbedding(m["dim"], m["rot"]["base"], rot_dim=m["rot"]["dims"])
     part = WindowAttention(width, m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"], window=m["mask"]["size"], pos_enc=pe,
-                           interleaved=sigmoid, qk_unit_eps=eps if sigmoid else None, keep_first=m["mask"].get("keep_first", 0) if sigmoid else 0,
+                           interleaved=sigmoid, qk_unit_eps=eps if sigmoid else None, keep_first=m["mask"].get("keep_first", 0),
                            sink=not sigmoid, sigmoid_weights=sigmoid)
     return part, pe
 
@@ -226,7 +226,7 @@ def test_attention_with_sigmoid_weights_and_kept_first_positions_alone(dtype, H,
 @pytest.mark.parametrize("H,G,dk,dv,size,dims,keep", ATT_SIZES)
 def test_attention_with_a_sink_alone(dtype, H, G, dk, dv, size, dims, keep, portion_kernel):
     width = 56
-    m = att(H, G, dk, dv, 2.0 / math.sqrt(dk), size, dims, base=300.0)
+    m = att(H, G, dk, dv, 2.0 / math.sqrt(dk), size, dims, base=300.0, keep=keep if H % 2 else None)    # kept positions go with a softmax too
     part, pe = attention_part(width, m, False)
     t = {}
     draw_attention(np.random.default_rng(H * dk + size), m, width, "", t, False)
