@@ -76,6 +76,27 @@ class stream_scope:
         return False
 
 
+class on_stream:
+    """Within the scope every op launches on ``stream`` (a ``torch.cuda.Stream``), whatever torch's current
+    stream is: for a part that runs two independent chains of kernels side by side.  The caller orders the two
+    streams (``wait_stream``) before and after; torch's own current stream, and with it where scratch memory is
+    allocated, stays as it is."""
+
+    def __init__(self, stream):
+        self._handle = ctypes.c_void_p(stream.cuda_stream)
+
+    def __enter__(self):
+        global _STREAM
+        self._outer = _STREAM
+        _STREAM = self._handle
+        return self
+
+    def __exit__(self, *exc):
+        global _STREAM
+        _STREAM = self._outer
+        return False
+
+
 def _dev(*ts):
     for t in ts:
         if t is not None and not t.is_cuda:

@@ -517,8 +517,35 @@ class TwoMixers(Mixer):
     def graph_safe(self) -> bool:
         return getattr(self.left, "graph_safe", True) and getattr(self.right, "graph_safe", True)
 
+    # Steps with prompt portions, launched eagerly: the halves are independent between the two products, and the
+    # right half's walk through its state is a chain that leaves most of the chip idle, so the left half's kernels
+    # run beside it on a second stream (of the default priority).  Not inside a graph capture, and not for steps
+    # of single tokens, which replay graphs.
+    TWO_STREAMS = True
+    TWO_STREAMS_IN_GRAPHS = True
+    _side_streams: Dict[object, object] = {}
+
+    def _side_stream(self, ctx):
+        if not TwoMixers.TWO_STREAMS or not hasattr(self.rt.ops, "on_stream") or self.rt.device.type != "cuda":
+            return None
+        if (ctx.max_q_len <= 1 or torch.cuda.is_current_stream_capturing()) and not TwoMixers.TWO_STREAMS_IN_GRAPHS:
+            return None
+        key = (self.rt.device.type, self.rt.device.index)
+        if key not in TwoMixers._side_streams:
+            TwoMixers._side_streams[key] = torch.cuda.Stream(device=self.rt.device)
+        return TwoMixers._side_streams[key]
+
     def forward(self, ctx, normed, cache) -> torch.Tensor:
         proj, act = self.set.project(ctx, normed)
-        self.left.core(ctx, self.set.views(0, proj), self.set.act_view(0, act), cache.kv)
+        side = self._side_stream(ctx)
+        if side is None:
+            self.left.core(ctx, self.set.views(0, proj), self.set.act_view(0, act), cache.kv)
+            self.right.core(ctx, self.set.views(1, proj), self.set.act_view(1, act), cache.state)
+            return self.set.output(ctx, act)
+        main = torch.cuda.current_stream(self.rt.device)
+        side.wait_stream(main)                           # the projections are there
+        with self.rt.ops.on_stream(side):
+            self.left.core(ctx, self.set.views(0, proj), self.set.act_view(0, act), cache.kv)
         self.right.core(ctx, self.set.views(1, proj), self.set.act_view(1, act), cache.state)
+        main.wait_stream(side)                           # both halves' activations are there
         return self.set.output(ctx, act)

@@ -556,6 +556,28 @@ def test_a_batch_gives_what_each_request_gives_alone(tdirs, name):
 
 
 @pytest.mark.parametrize("name", ["A", "B"])
+def test_the_halves_on_two_streams_give_the_same_bits(tdirs, name):
+    """The halves of a mixer of two run side by side on two streams; one after the other on one stream they
+    leave the same logits, bit for bit, in prompt portions and in single tokens."""
+    from rustinfer_amd.engine import StepEntry
+    from rustinfer_amd.parts import TwoMixers
+    toks = random_requests(CONFIGS[name]["vocab"], (150,), 33)["r0"]
+    keep = TwoMixers.TWO_STREAMS
+    outs = []
+    try:
+        for flag in (True, False):
+            TwoMixers.TWO_STREAMS = flag
+            eng = engine_for(tdirs[name], "bfloat16", name)
+            got = [eng.step([StepEntry("r0", toks[:100], list(range(100)))])]
+            got += [eng.step([StepEntry("r0", toks[100:120], list(range(20)))])]
+            got += [eng.step([StepEntry("r0", [t], [0])]) for t in toks[120:]]
+            outs.append(torch.cat([g.float().cpu() for g in got]))
+    finally:
+        TwoMixers.TWO_STREAMS = keep
+    assert torch.equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
 def test_long_decoding(tdirs, plain, name):
     """Twenty tokens of prompt and 280 single tokens: the windows pass over decoded tokens and give their pages
     back (not those of the kept positions), states, convolution inputs and shifted rows are carried 280 times."""
