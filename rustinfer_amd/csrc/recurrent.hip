@@ -60,6 +60,7 @@ struct ScanArgs {
     // w0 = A [H], ab = dt_bias [H]; kv_group heads share a head of r and k; r is multiplied by q_scale
     int gate_bf16, kv_group;
     float q_scale;
+    int decay_bf16;      // the dtype of al where it differs from wl's (the decays' inputs may stay 32-bit)
     // the channel forms: al holds the decays' inputs ([T][>= H dk], or [T][>= H] for a decay a head) in the gates'
     // dtype; ab their bias; w0 = A [H] where the form has one; decay_c = 1 / tau; skip [H] or null
     const float* skip;
@@ -177,12 +178,12 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                     raw_w[i][e] = on ? ld_f32(wlp + t * a.wl_stride + c) : 0.f;
                     raw_a[i][e] = on ? ld_f32(alp + t * a.al_stride + c) : 0.f;
                 }
-                if (CHAN_IN) raw_w[i][e] = on ? ld_gate(a.al, t * a.al_stride + h * dk + idx, a.gate_bf16) : 0.f;
+                if (CHAN_IN) raw_w[i][e] = on ? ld_gate(a.al, t * a.al_stride + h * dk + idx, a.decay_bf16) : 0.f;
             }
             if (GATED || VAR == 2) {
                 const size_t t = (size_t)(t_lo + c0 + (tt < nc ? tt : 0));
                 if (GATED) raw_gb[i] = ld_gate(a.wl, t * a.wl_stride + h, a.gate_bf16);
-                if (!CHAN_IN) raw_ga[i] = ld_gate(a.al, t * a.al_stride + h, a.gate_bf16);
+                if (!CHAN_IN) raw_ga[i] = ld_gate(a.al, t * a.al_stride + h, a.decay_bf16);
             }
         }
 #pragma unroll
@@ -467,7 +468,7 @@ extern "C" int ri_linear_scan(
     a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
     a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = silu_in; a.unit_eps = unit_eps; a.decay_c = decay_c;
     a.rot_cos = rot_cos; a.rot_sin = rot_sin; a.rot = rot_cos ? rot : 0; a.k_scale = k_scale;
-    a.gate_bf16 = 0; a.kv_group = 1; a.q_scale = 1.f; a.skip = nullptr;
+    a.gate_bf16 = 0; a.kv_group = 1; a.q_scale = 1.f; a.skip = nullptr; a.decay_bf16 = 0;
     int rc;
 #define RI_SCAN(TT, DD) (R == 8 ? launch_scan<TT, DD, 8>(a, num_rows, stream) : launch_scan<TT, DD, 16>(a, num_rows, stream))
     if (dtype == RI_F32) rc = delta ? RI_SCAN(float, true) : RI_SCAN(float, false);
@@ -508,7 +509,7 @@ extern "C" int ri_gated_delta_scan(
     a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
     a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = 0; a.unit_eps = unit_eps; a.decay_c = 0.f;
     a.rot_cos = nullptr; a.rot_sin = nullptr; a.rot = 0; a.k_scale = 1.f;
-    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale; a.skip = nullptr;
+    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale; a.skip = nullptr; a.decay_bf16 = a.gate_bf16;
     const int rc = R == 8 ? launch_scan<float, true, 8, true>(a, num_rows, stream) : launch_scan<float, true, 16, true>(a, num_rows, stream);
     if (rc) return rc;
     RI_LAUNCHED("ri_gated_delta_scan");
@@ -516,15 +517,16 @@ extern "C" int ri_gated_delta_scan(
 }
 
 // The channel-gated form of the walk: ri_gated_delta_scan with a decay for every key channel.  gl [T, >= H dk]
-// holds the decays' inputs in gate_dtype (as bl [T, >= H]), dt_bias [H dk] and A [H] are 32-bit:
+// holds the decays' inputs in decay_dtype (bl [T, >= H] in gate_dtype), dt_bias [H dk] and A [H] are 32-bit:
 // g = exp(-A_h softplus(gl + dt_bias)) over heads x dk.
 extern "C" int ri_channel_delta_scan(
         const float* q, int q_stride, const float* k, int k_stride, const float* v, int v_stride,
-        const void* bl, int bl_stride, const void* gl, int gl_stride, int gate_dtype,
+        const void* bl, int bl_stride, const void* gl, int gl_stride, int gate_dtype, int decay_dtype,
         const float* A, const float* dt_bias, float unit_eps, float q_scale,
         float* state, int num_slots, float* out, int out_stride,
         const int* cu_q, const int* q_start, const int* slots, int num_rows, int T,
         int H, int Hk, int dk, int dv, hipStream_t stream) {
+    RI_REQUIRE(decay_dtype == RI_F32 || decay_dtype == RI_BF16, "ri_channel_delta_scan: unknown dtype %d", decay_dtype);
     RI_REQUIRE(H > 0 && Hk > 0 && H % Hk == 0 && dk > 0 && dv > 0 && dk <= 256, "ri_channel_delta_scan: bad sizes H=%d Hk=%d dk=%d dv=%d (dk <= 256)", H, Hk, dk, dv);
     RI_REQUIRE(num_rows >= 0 && T >= 0 && num_slots > 0, "ri_channel_delta_scan: bad counts");
     RI_REQUIRE(q_stride >= Hk * dk && k_stride >= Hk * dk && v_stride >= H * dv && out_stride >= H * dv && bl_stride >= H && gl_stride >= H * dk,
@@ -543,7 +545,7 @@ extern "C" int ri_channel_delta_scan(
     a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
     a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = 0; a.unit_eps = unit_eps; a.decay_c = 0.f;
     a.rot_cos = nullptr; a.rot_sin = nullptr; a.rot = 0; a.k_scale = 1.f;
-    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale; a.skip = nullptr;
+    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale; a.skip = nullptr; a.decay_bf16 = decay_dtype == RI_BF16;
     const int rc = R == 8 ? launch_scan<float, true, 8, true, 1>(a, num_rows, stream) : launch_scan<float, true, 16, true, 1>(a, num_rows, stream);
     if (rc) return rc;
     RI_LAUNCHED("ri_channel_delta_scan");
@@ -582,7 +584,7 @@ extern "C" int ri_decay_scan(
     a.cu_q = cu_q; a.q_start = q_start; a.slots = slots;
     a.H = H; a.dk = dk; a.dv = dv; a.P = P; a.silu_in = 0; a.unit_eps = 0.f; a.decay_c = inv_tau;
     a.rot_cos = nullptr; a.rot_sin = nullptr; a.rot = 0; a.k_scale = 1.f;
-    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale; a.skip = skip;
+    a.gate_bf16 = gate_dtype == RI_BF16; a.kv_group = H / Hk; a.q_scale = q_scale; a.skip = skip; a.decay_bf16 = a.gate_bf16;
     int rc;
 #define RI_DSCAN(TT, VV) (R == 8 ? launch_scan<TT, false, 8, false, VV>(a, num_rows, stream) : launch_scan<TT, false, 16, false, VV>(a, num_rows, stream))
     if (dtype == RI_F32) rc = mode == 1 ? RI_DSCAN(float, 1) : RI_DSCAN(float, 2);

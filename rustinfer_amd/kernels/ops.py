@@ -1481,7 +1481,7 @@ def channel_delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta_i
                        H: int, Hk: int, dk: int, dv: int, unit_eps: float = 1e-6, q_scale: float = 1.0) -> None:
     """``gated_delta_scan`` with a decay for every key channel: ``S <- diag(g) S; u = beta (v - S^T k);
     S <- S + k u^T; out = S^T q`` with ``g = exp(-A_h softplus(decay_in + dt_bias))`` laid out heads x dk
-    (``decay_in [T, H dk]`` activations, ``dt_bias [H dk]`` and ``A [H]`` 32-bit) and ``beta = sigmoid(beta_in)``,
+    (``decay_in [T, H dk]`` activations or 32-bit, ``dt_bias [H dk]`` and ``A [H]`` 32-bit) and ``beta = sigmoid(beta_in)``,
     ``beta_in [T, H]``.  q, k ``[T, Hk dk]`` and v ``[T, H dv]`` 32-bit; q and k are divided by
     ``sqrt(|.|^2 + unit_eps)``, q also times ``q_scale``."""
     _dev(q, k, v, beta_in, decay_in, A, dt_bias, state, out)
@@ -1491,14 +1491,14 @@ def channel_delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta_i
     if tuple(q.shape) != (T, Hk * dk) or tuple(k.shape) != (T, Hk * dk) or tuple(v.shape) != (T, H * dv) \
             or any(t.dtype != torch.float32 for t in (q, k, v)):
         raise KernelError("channel_delta_scan: 32-bit q, k [T, Hk dk] and v [T, H dv] expected")
-    if tuple(beta_in.shape) != (T, H) or tuple(decay_in.shape) != (T, H * dk) or beta_in.dtype != decay_in.dtype:
-        raise KernelError("channel_delta_scan: beta_in [T, H] and decay_in [T, H dk] of one dtype expected")
+    if tuple(beta_in.shape) != (T, H) or tuple(decay_in.shape) != (T, H * dk):
+        raise KernelError("channel_delta_scan: beta_in [T, H] and decay_in [T, H dk] expected")
     _scan_common(state, out, ctx, H, dk, dv, T, "channel_delta_scan")
     _f32_vec(A, H, "channel_delta_scan: A")
     _f32_vec(dt_bias, H * dk, "channel_delta_scan: dt_bias")
     _check(_lib().ri_channel_delta_scan(
         _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(beta_in), beta_in.stride(0),
-        _ptr(decay_in), decay_in.stride(0), _dt(beta_in), _ptr(A), _ptr(dt_bias), ctypes.c_float(unit_eps),
+        _ptr(decay_in), decay_in.stride(0), _dt(beta_in), _dt(decay_in), _ptr(A), _ptr(dt_bias), ctypes.c_float(unit_eps),
         ctypes.c_float(q_scale), _ptr(state), state.shape[0], _ptr(out), out.stride(0), _ptr(ctx.cu_q), _ptr(ctx.q_start),
         _ptr(ctx.state_slots), ctx.num_rows, T, H, Hk, dk, dv, _stream()))
 

@@ -350,7 +350,7 @@ class ChannelGatedDeltaRule(ProjectedPart, Mixer):
         mixed = ws.get("gdelta.conv", T, self.conv_channels, torch.float32)
         ops.short_conv([proj[n["q"]], proj[n["k"]], proj[n["v"]]], self.conv_weights,
                        cache.extra["conv"] if self.conv_taps > 1 else None, mixed, ctx, self.conv_taps, silu=True)
-        decay_in = ws.get("gdelta.decay_in", T, H * dk, self.rt.dtype)
+        decay_in = ws.get("gdelta.decay_in", T, H * dk, torch.float32)      # the decays' inputs leave their product unrounded
         self.a2.forward(proj[n["a1"]], decay_in)
         gate_in = ws.get("gdelta.gate_in", T, H * dv, self.rt.dtype)
         self.g2.forward(proj[n["g1"]], gate_in)
@@ -407,7 +407,7 @@ class GatedLinearAttention(ProjectedPart, Mixer):
     def core(self, ctx, proj, act, cache) -> None:
         ops, n, ws = self.rt.ops, self.names, ctx.workspace
         T, H, dk, dv = act.shape[0], self.num_heads, self.head_dim, self.v_head_dim
-        decay_in = ws.get("gla.decay_in", T, H * dk, self.rt.dtype)
+        decay_in = ws.get("gla.decay_in", T, H * dk, torch.float32)         # the decays' inputs leave their product unrounded
         self.a2.forward(proj[n["a1"]], decay_in)
         o = ws.get("scan.o", T, H * dv, torch.float32)
         ops.decay_scan("channel", proj[n["q"]], proj[n["k"]], proj[n["v"]], decay_in, self.decay_bias, cache.state, o, ctx,
