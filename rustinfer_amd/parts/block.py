@@ -517,10 +517,11 @@ class TwoMixers(Mixer):
     def graph_safe(self) -> bool:
         return getattr(self.left, "graph_safe", True) and getattr(self.right, "graph_safe", True)
 
-    # Steps with prompt portions, launched eagerly: the halves are independent between the two products, and the
-    # right half's walk through its state is a chain that leaves most of the chip idle, so the left half's kernels
-    # run beside it on a second stream (of the default priority).  Not inside a graph capture, and not for steps
-    # of single tokens, which replay graphs.
+    # The halves are independent between the two products, and the right half's walk through its state is a chain
+    # that leaves most of the chip idle, so the left half's kernels run beside it on a second stream (of the
+    # default priority) that waits for the in-product and is waited for before the out-product.  Inside a graph
+    # capture the same fork and join make two branches of the graph (TWO_STREAMS_IN_GRAPHS; steps of single tokens
+    # go the same way, captured or not).
     TWO_STREAMS = True
     TWO_STREAMS_IN_GRAPHS = True
     _side_streams: Dict[object, object] = {}
