@@ -76,6 +76,9 @@ __device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log
 __device__ __forceinline__ float expf_(float z) { return __expf(z); }
 __device__ __forceinline__ float sigmoidf_(float z) { return __fdividef(1.f, 1.f + __expf(-z)); }
 __device__ __forceinline__ float siluf_(float z) { return __fdividef(z, 1.f + __expf(-z)); }
+// softplus on the hardware's 2^x and log2 (an absolute error of a few 1e-8 where the result is small): for the
+// decays of every key channel, which the staging makes dk at a time
+__device__ __forceinline__ float softplus_fast(float z) { return z > 20.f ? z : __logf(1.f + __expf(z)); }
 
 // Sum over the P adjacent lanes that share a column (P a power of two up to 16), every lane
 // getting the same bits: exchanges inside a quad, between the quads of half a row, between the
@@ -220,7 +223,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                         if (VAR == 1) {
                             // sigmoid(z)^(1/tau) = exp(-softplus(-z) / tau)
                             r = raw_r[i][e] * a.q_scale; k = raw_k[i][e];
-                            w = expf(-softplusf_(-(raw_w[i][e] + a.ab[h * dk + idx])) * a.decay_c);
+                            w = expf_(-softplus_fast(-(raw_w[i][e] + a.ab[h * dk + idx])) * a.decay_c);
                         } else {
                             r = raw_r[i][e]; k = dt * raw_k[i][e]; w = dec;
                         }
@@ -242,7 +245,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                     if (idx >= DKP) continue;
                     const bool in = idx < dk;
                     const float u = in ? raw_k[i][e] * inv_k : 0.f;
-                    const float g = in ? expf(-rate * softplusf_(raw_w[i][e] + a.ab[h * dk + idx])) : 0.f;
+                    const float g = in ? expf_(-rate * softplus_fast(raw_w[i][e] + a.ab[h * dk + idx])) : 0.f;
                     rs[tt * DKP + idx] = in ? raw_r[i][e] * inv_q : 0.f;
                     us[tt * DKP + idx] = g * u; ks[tt * DKP + idx] = beta * u;
                     aus[tt * DKP + idx] = beta * u; ws[tt * DKP + idx] = g;
@@ -328,8 +331,9 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
         const float* aus = us + SC_CH * DKP;
         const float* ws = VDEC ? us : aus + SC_CH * DKP;
         const float* vs = buf + NA * SC_CH * DKP;
-#pragma unroll 4
-        for (int tt = 0; tt < nc; ++tt) {
+        // a token of the stretch; a whole stretch is unrolled, so that its reads from LDS are all asked for before
+        // the first is used (a wave alone on its SIMD waits out every read it asks for late)
+        auto walk = [&](int tt) {
             const float vv = vs[tt * CPB + jc];
             const int base = tt * DKP + pl * R;
             if (DELTA) {
@@ -377,6 +381,13 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
             o = group_sum(o, P);
             if (VDEC) o = fmaf(skip, vv, o);
             if (pl == 0 && col_ok) a.out[(size_t)(t_lo + c0 + tt) * a.out_stride + h * dv + j] = o;
+        };
+        if (nc == SC_CH) {
+#pragma unroll
+            for (int tt = 0; tt < SC_CH; ++tt) walk(tt);
+        } else {
+#pragma unroll 1
+            for (int tt = 0; tt < nc; ++tt) walk(tt);
         }
     }
 #pragma unroll
