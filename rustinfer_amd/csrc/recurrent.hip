@@ -211,8 +211,8 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
             if (VDEC) {
                 float dt = 0.f, dec = 0.f;
                 if (VAR == 2) {
-                    dt = softplusf_(raw_ga[i] + a.ab[h]);
-                    dec = expf(-a.w0[h] * dt);
+                    dt = softplus_fast(raw_ga[i] + a.ab[h]);
+                    dec = expf_(-a.w0[h] * dt);
                 }
 #pragma unroll
                 for (int e = 0; e < SC_EPL; ++e) {
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(NW * 64) void linear_scan_kernel(const ScanArgs a) 
                 sk = wave_sum_rows(sk);
                 sq = wave_sum_rows(sq);
                 const float inv_k = 1.f / sqrtf(sk + a.unit_eps), inv_q = a.q_scale / sqrtf(sq + a.unit_eps);
-                const float beta = 1.f / (1.f + expf(-raw_gb[i]));
+                const float beta = sigmoidf_(raw_gb[i]);
                 const float rate = a.w0[h];
 #pragma unroll
                 for (int e = 0; e < SC_EPL; ++e) {
